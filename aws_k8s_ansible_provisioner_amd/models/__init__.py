@@ -11,6 +11,10 @@ def model_class(cfg: ModelConfig):
         from .puputar import PuputarLM
 
         return PuputarLM
+    if cfg.arch == "sazepel":
+        from .sazepel import SazepelLM
+
+        return SazepelLM
     from .transformer import DecoderLM
 
     return DecoderLM

@@ -18,7 +18,7 @@ from typing import Optional
 class ModelConfig:
     name: str
     hf_id: str
-    arch: str  # "qwen3" | "llama" | "mixtral" | "qwen3_moe" | "bidetar" | "puputar" (LayeredConfig)
+    arch: str  # "qwen3" | "llama" | "mixtral" | "qwen3_moe" | "bidetar" | "puputar" | "sazepel" (LayeredConfig)
     vocab_size: int
     hidden_size: int
     intermediate_size: int
@@ -123,6 +123,56 @@ class AttentionSpec:
     sink: bool = True
     gate: bool = True
     shared_kv: bool = True
+    # head_norm: q and k are divided by their root mean square per head (no weights);
+    # v_norm: so are the cached values; talk: the heads' softmax weights are mixed by a learned
+    # [H, H] matrix before they meet the values; gate_per "element": one sigmoid gate per
+    # output entry instead of one per head
+    head_norm: bool = False
+    v_norm: bool = False
+    talk: bool = False
+    gate_per: str = "head"
+
+
+@dataclasses.dataclass
+class RetentionSpec:
+    """Linear attention with a fixed decay per head and no softmax: per head a state
+    S [dim, vdim] (fp32, one per live sequence) with S_t = decay_h S_{t-1} + k_t v_t^T and
+    o_t = S_t^T q_t; rotary positions on q and k in the rotate-half layout (dimension i pairs
+    with i + dims/2); k scaled by dim^-1/2; each head's output divided by its root mean square
+    and gated by silu of a projection of the mixer's input."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: tuple
+    rot: Optional[RotarySpec] = None
+    # sizing fields shared with AttentionSpec: a retention mixer caches no keys
+    kv_heads: int = 0
+    chunk: int = 0
+    window: int = 0
+
+    @property
+    def state_floats(self) -> int:
+        return self.heads * self.dim * self.vdim
+
+
+@dataclasses.dataclass
+class ParallelMixerSpec:
+    """Two mixers side by side on the same input; the layer's mixer output is half the sum of
+    their outputs, each RMS-normed over the model width with a weight vector of its own."""
+    left: AttentionSpec
+    right: RetentionSpec
+
+    @property
+    def heads(self) -> int:
+        return max(self.left.heads, self.right.heads)
+
+    @property
+    def kv_heads(self) -> int:
+        return self.left.kv_heads
+
+    @property
+    def dim(self) -> int:
+        return max(self.left.dim, self.left.vdim)
 
 
 @dataclasses.dataclass
@@ -170,6 +220,9 @@ class RouterSpec:
     identity: int = 0
     groups: int = 1
     keep: int = 1
+    # "corrected": the rule above.  "logits": the `top` largest of (router h + bias) win and
+    # their weights are the softmax over the winners' logits only
+    kind: str = "corrected"
 
     @property
     def outputs(self) -> int:
@@ -180,15 +233,15 @@ class RouterSpec:
 class MlpSpec:
     kind: str   # "dense": down(act(up h)) | "moe": routed experts of that form
     ff: int
-    act: str = "relu2"              # "relu2" | "xielu" (two learned numbers per layer)
+    act: str = "relu2"              # "relu2" | "xielu" (two learned numbers per layer) | "swiglu"
     bias: bool = False
     router: Optional[RouterSpec] = None
 
 
 @dataclasses.dataclass
 class LayerSpec:
-    type: str                       # which mixer: "attention" | "latent_attention[_2]"
-    mixer: object                   # AttentionSpec | LatentAttentionSpec
+    type: str                       # "attention" | "latent_attention[_2]" | "retention" | "parallel"
+    mixer: object                   # AttentionSpec | LatentAttentionSpec | RetentionSpec | ParallelMixerSpec
     mlp: Optional[MlpSpec] = None   # None: the layer has no feed-forward
 
 
@@ -204,6 +257,7 @@ class LayeredConfig(ModelConfig):
     embed_scale: float = 1.0
     residual_mult: float = 1.0
     norm_groups: int = 1            # RMS norms of the stream run in this many equal parts
+    logit_scale: float = 1.0        # logits = head x * logit_scale
 
     def layer_runs(self) -> list:
         """Indices into layer_specs in execution order."""
@@ -220,15 +274,22 @@ class LayeredConfig(ModelConfig):
             m = self.layer_specs[i].mixer
             if isinstance(m, LatentAttentionSpec):
                 n += 0 if m.kv_from is not None else m.cache_dim * es
+            elif isinstance(m, RetentionSpec):
+                pass
+            elif isinstance(m, ParallelMixerSpec):
+                n += m.left.kv_heads * (m.left.dim + m.left.vdim) * es
             else:
                 n += 2 * m.kv_heads * m.dim * es
         return n
 
     def num_params(self) -> int:
         d = self.hidden_size
-        n = 2 * self.vocab_size * d + d
+        n = 2 * self.vocab_size * d + (2 if self.arch == "sazepel" else d)
         for ls in self.layer_specs:
             m = ls.mixer
+            if isinstance(m, (RetentionSpec, ParallelMixerSpec)):
+                n += _sazepel_layer_params(d, ls)
+                continue
             if isinstance(m, LatentAttentionSpec):
                 n += 3 * d + m.q_rank * (d + 1) + m.heads * (m.dim + m.rot_dim) * m.q_rank \
                     + m.heads * (m.dim + m.vdim) * m.kv_rank + m.gate_rows * d \
@@ -246,6 +307,21 @@ class LayeredConfig(ModelConfig):
             if ls.mlp is not None:
                 n += 2 * d * ls.mlp.ff
         return n
+
+
+def _sazepel_layer_params(d: int, ls: "LayerSpec") -> int:
+    def ret(r):
+        return d * r.heads * (2 * r.dim + 3 * r.vdim)
+
+    def att(a):
+        return d * (a.heads * (a.dim + 2 * a.vdim) + a.kv_heads * (a.dim + a.vdim)) + a.heads ** 2
+
+    m = ls.mixer
+    n = 2 + (ret(m) if isinstance(m, RetentionSpec) else att(m.left) + ret(m.right) + 2 * d)
+    if ls.mlp is not None:
+        e = ls.mlp.router.experts if ls.mlp.router else 1
+        n += 2 + 3 * d * ls.mlp.ff * e + (e * (d + 1) if ls.mlp.router else 0)
+    return n
 
 
 def bidetar_config(name: str, d: dict, max_position: int = 1 << 20) -> LayeredConfig:
@@ -355,6 +431,93 @@ def puputar_config(name: str, d: dict, max_position: int = 1 << 20) -> LayeredCo
     return cfg
 
 
+def _sazepel_retention(m: dict) -> RetentionSpec:
+    rot = m.get("rot")
+    rs = RotarySpec(int(rot["dims"]), float(rot["base"])) if rot and int(rot["dims"]) > 0 else None
+    spec = RetentionSpec(heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                         decay=tuple(float(g) for g in m["decay"]), rot=rs)
+    if len(spec.decay) != spec.heads or not all(0.0 < g <= 1.0 for g in spec.decay):
+        raise ValueError("Sazepel: one decay in (0, 1] per retention head")
+    if rs is not None and (rs.dims % 2 or rs.dims > spec.dim):
+        raise ValueError("Sazepel: rot.dims must be even and at most dim")
+    return spec
+
+
+def _sazepel_attention(m: dict) -> AttentionSpec:
+    spec = AttentionSpec(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]),
+                         vdim=int(m["vdim"]), scale=float(m["scale"]), rot=None, sink=False,
+                         gate=True, shared_kv=False, head_norm=True, v_norm=True, talk=True,
+                         gate_per="element")
+    if spec.heads % spec.kv_heads:
+        raise ValueError("Sazepel: heads must be a multiple of kv_heads")
+    return spec
+
+
+def sazepel_config(name: str, d: dict, max_position: int = 1 << 20) -> LayeredConfig:
+    """A Sazepel config.json: sequential layers (a norm before and after each sublayer, every
+    norm weight one number), mixers "retention" (decayed linear attention with a recurrent
+    state) or "parallel" (a softmax attention with head-mixed weights beside a retention),
+    routed SwiGLU feed-forwards (or none), scaled logits."""
+    specs = []
+    for ly in d["layers"]:
+        if ly["type"] == "retention":
+            mixer = _sazepel_retention(ly["mixer"])
+        elif ly["type"] == "parallel":
+            mixer = ParallelMixerSpec(_sazepel_attention(ly["mixer"]["left"]),
+                                      _sazepel_retention(ly["mixer"]["right"]))
+        else:
+            raise ValueError(f"Sazepel: unknown mixer type {ly['type']!r}")
+        ml = ly.get("mlp")
+        mlp = None
+        if ml is not None:
+            if ml.get("kind") != "moe":
+                raise ValueError(f"Sazepel: unknown feed-forward kind {ml.get('kind')!r}")
+            rt = ml["router"]
+            router = RouterSpec(experts=int(rt["experts"]), top=int(rt["top"]), kind="logits")
+            if not 1 <= router.top <= router.experts:
+                raise ValueError(f"Sazepel: bad router {rt}")
+            mlp = MlpSpec("moe", int(ml["expert"]["ff"]), act="swiglu", router=router)
+        specs.append(LayerSpec(ly["type"], mixer, mlp))
+    cfg = LayeredConfig(
+        name=name, hf_id=name, arch="sazepel", vocab_size=int(d["vocab"]),
+        hidden_size=int(d["width"]),
+        intermediate_size=max([ls.mlp.ff for ls in specs if ls.mlp is not None] or [0]),
+        num_layers=len(specs), num_heads=max(ls.mixer.heads for ls in specs),
+        num_kv_heads=max([ls.mixer.kv_heads for ls in specs] + [1]),
+        head_dim=max(ls.mixer.dim for ls in specs), rms_eps=float(d["norm"]["eps"]),
+        max_position=max_position, bos_id=0, eos_id=-1, layer_specs=specs,
+        logit_scale=float(d.get("logit_scale", 1.0)))
+    return cfg
+
+
+def sazepel_dict(width: int, layers: list, vocab: int = 32000, eps: float = 1e-6,
+                 logit_scale: float = 1.0) -> dict:
+    """A Sazepel config.json dictionary from short layer dicts (random-init benchmarks and
+    tests).  A layer gives `ret` = (heads, dim, vdim) and optionally `att` = (heads, kv_heads,
+    dim, vdim) (then the layer is "parallel"), `experts` / `expert_ff` / `top` (else no
+    feed-forward), and optional decay (list), rot_dims, base, scale."""
+    out = []
+    for ly in layers:
+        H, D, V = ly["ret"]
+        decay = ly.get("decay") or [1.0 - 2.0 ** (-5.0 - 5.0 * h / max(1, H - 1)) for h in range(H)]
+        ret = {"heads": H, "dim": D, "vdim": V, "decay": [float(g) for g in decay],
+               "rot": {"base": float(ly.get("base", 10000.0)), "dims": int(ly.get("rot_dims", D))}}
+        if "att" in ly:
+            h, g, dd, vv = ly["att"]
+            mixer = {"left": {"heads": h, "kv_heads": g, "dim": dd, "vdim": vv,
+                              "scale": float(ly.get("scale", dd ** -0.5))}, "right": ret}
+            kind = "parallel"
+        else:
+            mixer, kind = ret, "retention"
+        mlp = None
+        if ly.get("experts"):
+            mlp = {"kind": "moe", "expert": {"ff": ly["expert_ff"]},
+                   "router": {"experts": ly["experts"], "top": ly["top"]}}
+        out.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Sazepel", "layers": out, "logit_scale": logit_scale,
+            "norm": {"eps": eps}, "vocab": vocab, "width": width}
+
+
 def puputar_dict(width: int, layers: list, vocab: int = 32000, eps: float = 1e-6,
                  norm_groups: int = 1) -> dict:
     """A Puputar config.json dictionary from short layer tuples (random-init benchmarks and
@@ -385,7 +548,8 @@ def puputar_dict(width: int, layers: list, vocab: int = 32000, eps: float = 1e-6
 
 
 # config.json readers of designs that do not use the HF key set, by their "architecture" value
-_NATIVE_READERS = {"Bidetar": bidetar_config, "Puputar": puputar_config}
+_NATIVE_READERS = {"Bidetar": bidetar_config, "Puputar": puputar_config,
+                   "Sazepel": sazepel_config}
 
 _REGISTRY: dict[str, ModelConfig] = {}
 

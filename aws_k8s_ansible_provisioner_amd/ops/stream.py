@@ -632,3 +632,245 @@ def moe_combine(out: torch.Tensor, y: torch.Tensor, inv: Optional[torch.Tensor],
         real = (w * (ids < experts))[:, :, None]
         acc = (y.float()[inv.long().clamp(min=0, max=y.shape[0] - 1)] * real).sum(dim=1)
     out.copy_(acc + ident * h.float())
+
+
+# ----------------------------------------------------------------------------- sandwich norms
+def _w(w: torch.Tensor) -> torch.Tensor:
+    return w.float()
+
+
+def stream_post_norm_add_norm(x: torch.Tensor, ya: torch.Tensor, yb: Optional[torch.Tensor],
+                              wa: Optional[torch.Tensor], wb: Optional[torch.Tensor],
+                              post_w: torch.Tensor, next_w: torch.Tensor, eps: float,
+                              out: torch.Tensor, fresh: bool = False) -> None:
+    """The residual update of a sublayer whose OUTPUT is normed, fused with the norm that feeds
+    the next sublayer:  m = ya, or with two branches m = (rms(ya) wa + rms(yb) wb) / 2;
+    x <- x + rms(m) post_w (fresh: x <- rms(m) post_w, x is not read);  out = rms(x) next_w.
+    rms(v) = v / sqrt(mean(v^2) + eps) over the row.  x fp32 [T, d] (the stream, updated in
+    place); ya / yb [T, d] in the activation type or fp32; every weight is fp32 with d entries
+    or ONE (a single number for all coordinates).  All arithmetic is fp32; out is rounded
+    once."""
+    if _native(x):
+        torch.ops.akap_stream.post_norm_add_norm(out, x, ya, yb, wa, wb, post_w, next_w,
+                                                 float(eps), bool(fresh))
+        return
+    m = ya.float()
+    if yb is not None:
+        m = 0.5 * (_rms(m, eps) * _w(wa) + _rms(yb.float(), eps) * _w(wb))
+    upd = _rms(m, eps) * _w(post_w)
+    if fresh:
+        x.copy_(upd)
+    else:
+        x.add_(upd)
+    out.copy_((_rms(x, eps) * _w(next_w)).to(out.dtype))
+
+
+# ----------------------------------------------------------------------------- head-mixed attention
+def head_norm_cache(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor,
+                    v_cache: torch.Tensor, slots: torch.Tensor, H: int, G: int, D: int, Dv: int,
+                    q_off: int, k_off: int, v_off: int, eps: float, norm_qk: bool = True,
+                    norm_v: bool = True) -> None:
+    """Per token t of the fused projection proj [T, N]: the H query heads
+    proj[t, q_off : q_off + H D] go to q_out [T, H, D], the G key heads (from k_off) to k_cache
+    [NB, G, BS, D] and the G value heads (from v_off, size Dv) to v_cache [NB, G, BS, Dv] at
+    slots[t] (-1: nothing is cached).  norm_qk / norm_v: each head is first divided by its own
+    root mean square (fp32, eps inside the root, no weights)."""
+    if _native(proj):
+        torch.ops.akap_stream.head_norm_cache(proj, q_out, k_cache, v_cache, slots, H, G, D, Dv,
+                                              q_off, k_off, v_off, float(eps), bool(norm_qk),
+                                              bool(norm_v))
+        return
+    T = proj.shape[0]
+    q = proj[:, q_off:q_off + H * D].float().view(T, H, D)
+    k = proj[:, k_off:k_off + G * D].float().view(T, G, D)
+    v = proj[:, v_off:v_off + G * Dv].float().view(T, G, Dv)
+    if norm_qk:
+        q, k = _rms(q, eps), _rms(k, eps)
+    if norm_v:
+        v = _rms(v, eps)
+    q_out.copy_(q.to(q_out.dtype))
+    BS = k_cache.shape[2]
+    ok = slots >= 0
+    sl = slots[ok].long()
+    k_cache[sl // BS, :, sl % BS] = k[ok].to(k_cache.dtype)
+    v_cache[sl // BS, :, sl % BS] = v[ok].to(v_cache.dtype)
+
+
+def talking_attention_parts(rows: int, kv_heads: int, max_len: int) -> int:
+    """Key partitions of a decode row of talking_attention: static in the batch size and the
+    model length (hipGraph-capturable); about four workgroups per CU, a partition never under
+    128 keys."""
+    max_parts = max(1, -(-max_len // 128))
+    return max(1, min(max_parts, 32, -(-1024 // max(1, rows * kv_heads))))
+
+
+def talking_attention_workspace(rows: int, H: int, G: int, Dv: int, parts: int, device):
+    """Partial state of the split form: (max, sum) per (row, partition, head) and the
+    unnormalised outputs of every (head, value head) pair, fp32."""
+    n = max(1, rows * parts)
+    return (torch.empty(n * H * 2, dtype=torch.float32, device=device),
+            torch.empty(n * H * G * Dv, dtype=torch.float32, device=device))
+
+
+def talking_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
+                      v_cache: torch.Tensor, block_tables: torch.Tensor, seq_lens: torch.Tensor,
+                      q_start: Optional[torch.Tensor], positions: torch.Tensor,
+                      talk: Optional[torch.Tensor], gate: Optional[torch.Tensor], scale: float,
+                      workspace=None, num_parts: int = 1) -> None:
+    """Causal softmax attention whose heads exchange their weights AFTER the softmax: with
+    P_g(t, j) = softmax_j(q[t, g] . k[j, g // (H / G)] * scale) over the keys j <= positions[t]
+    of row t's sequence, head h uses P'_h = sum_g talk[h, g] P_g on the values of ITS OWN
+    key/value head:  out[t, h Dv : (h + 1) Dv] = sum_j P'_h(t, j) v[j, h // (H / G)], times
+    sigmoid(gate[t, h Dv + i]) per entry when gate is given.  talk None: no mixing.
+    Row t belongs to sequence b with q_start[b] <= t < q_start[b + 1] (q_start None: row t is
+    sequence t); sequences with seq_lens[b] == 0 are padding and their rows are left unwritten.
+    q [T, H, D]; k_cache [NB, G, BS, D]; v_cache [NB, G, BS, Dv]; talk fp32 [H, H]; gate and
+    out are [T, H Dv] views that may be column slices of wider rows.  Scores, softmax, the
+    mixing and the gate are fp32.
+    The GPU kernel forms, for every head g, the unnormalised sums of ALL G value heads under
+    its weights (one pass over the keys with a running maximum), and mixes them at the end;
+    num_parts > 1 cuts the keys of a row into that many partitions, one workgroup each, merged,
+    mixed and gated by a second launch (workspace from talking_attention_workspace)."""
+    if _native(q):
+        ws_ml, ws_o = workspace if (workspace is not None and num_parts > 1) else (None, None)
+        torch.ops.akap_stream.talking_attention(out, q, k_cache, v_cache, block_tables, seq_lens,
+                                                q_start, positions, talk, gate, float(scale),
+                                                ws_ml, ws_o, num_parts if ws_ml is not None else 1)
+        return
+    T, H, D = q.shape
+    G, BS, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    rep = H // G
+    B = seq_lens.numel()
+    for b in range(B):
+        kv = int(seq_lens[b])
+        r0, r1 = (b, b + 1) if q_start is None else (int(q_start[b]), int(q_start[b + 1]))
+        if kv == 0 or r1 <= r0:
+            continue
+        nb = -(-kv // BS)
+        blocks = block_tables[b, :nb].long()
+        K = k_cache[blocks].permute(1, 0, 2, 3).reshape(G, nb * BS, D)[:, :kv].float()
+        V = v_cache[blocks].permute(1, 0, 2, 3).reshape(G, nb * BS, Dv)[:, :kv].float()
+        pos = positions[r0:r1].long()
+        ok = torch.arange(kv)[None, :] <= pos[:, None]
+        s = torch.einsum("thd,hjd->htj", q[r0:r1].float(), K.repeat_interleave(rep, dim=0)) * scale
+        P = torch.softmax(s.masked_fill(~ok[None], float("-inf")), dim=-1)
+        if talk is not None:
+            P = torch.einsum("hg,gtj->htj", talk.float(), P)
+        o = torch.einsum("htj,hjv->thv", P, V.repeat_interleave(rep, dim=0)).reshape(r1 - r0, H * Dv)
+        if gate is not None:
+            o = o * torch.sigmoid(gate[r0:r1].float())
+        out[r0:r1] = o.to(out.dtype)
+
+
+# ----------------------------------------------------------------------------- retention
+def rotate_half_(x: torch.Tensor, cs: torch.Tensor) -> torch.Tensor:
+    """x [T, H, D] (fp32) with its first cs.shape[1] dimensions rotated, dimension i paired
+    with i + dims/2, by the table rows cs [T, dims] = [cos | sin]."""
+    dims = cs.shape[1]
+    half = dims // 2
+    c, s = cs[:, None, :half], cs[:, None, half:]
+    u, v = x[..., :half].clone(), x[..., half:dims].clone()
+    x[..., :half] = u * c - v * s
+    x[..., half:dims] = v * c + u * s
+    return x
+
+
+def retention(out: torch.Tensor, proj: torch.Tensor, q_off: int, k_off: int, v_off: int,
+              g_off: int, state: torch.Tensor, seq_slot: torch.Tensor, positions: torch.Tensor,
+              q_start: Optional[torch.Tensor], cos_sin: Optional[torch.Tensor],
+              log2_decay: torch.Tensor, H: int, D: int, V: int, eps: float) -> None:
+    """Decayed linear attention with a recurrent state, for the token rows of a step.  Per
+    token t and head h, from the fused projection proj [T, N]: q, k = proj[t, q_off / k_off +
+    h D ...] (D entries), v = proj[t, v_off + h V ...], g = proj[t, g_off + h V ...] (V
+    entries).  q and k are rotated on their first cos_sin.shape[1] dimensions in the rotate-half
+    layout (i pairs with i + dims/2) by the angle row of positions[t]; k is scaled by D^-1/2;
+    S <- decay_h S + k v^T and o = S^T q with decay_h = 2^log2_decay[h]; o is divided by its
+    root mean square over V (eps inside the root) and multiplied by silu(g):
+    out[t, h V : (h + 1) V].  The state S [D, V] (fp32) of a sequence lives in
+    state[slot, h]: the rows of sequence b are [q_start[b], q_start[b + 1]) (q_start None: row
+    t is a sequence of its own), its slot is seq_slot of its first row (-1: padding, nothing
+    is read or written); it starts from zeros when its first row has position 0, else from
+    what an earlier step left in the slot, and the state after its last row is written back.
+    Rotation, decay, state, the output norm and the gate are fp32.  out may be a column slice
+    of wider rows."""
+    if _native(proj):
+        torch.ops.akap_stream.retention(out, proj, q_off, k_off, v_off, g_off, state, seq_slot,
+                                        positions, q_start, cos_sin, log2_decay, H, D, V,
+                                        float(eps))
+        return
+    T = proj.shape[0]
+    q = proj[:, q_off:q_off + H * D].float().reshape(T, H, D).clone()
+    k = proj[:, k_off:k_off + H * D].float().reshape(T, H, D).clone()
+    v = proj[:, v_off:v_off + H * V].float().reshape(T, H, V)
+    g = proj[:, g_off:g_off + H * V].float().reshape(T, H, V)
+    if cos_sin is not None:
+        cs = cos_sin[positions.long()]
+        rotate_half_(q, cs)
+        rotate_half_(k, cs)
+    k = k * (D ** -0.5)
+    decay = torch.exp2(log2_decay.float())[:, None, None]
+    B = T if q_start is None else q_start.numel() - 1
+    o = torch.zeros(T, H, V, dtype=torch.float32)
+    for b in range(B):
+        r0, r1 = (b, b + 1) if q_start is None else (int(q_start[b]), int(q_start[b + 1]))
+        if r1 <= r0 or int(seq_slot[r0]) < 0:
+            continue
+        slot = int(seq_slot[r0])
+        S = state[slot].float().clone() if int(positions[r0]) > 0 else \
+            torch.zeros(H, D, V, dtype=torch.float32)
+        for t in range(r0, r1):
+            S = decay * S + k[t][:, :, None] * v[t][:, None, :]
+            o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+        state[slot] = S
+        on = _rms(o[r0:r1], eps) * torch.nn.functional.silu(g[r0:r1])
+        out[r0:r1] = on.reshape(r1 - r0, H * V).to(out.dtype)
+
+
+# ----------------------------------------------------------------------------- logit-top-k routing
+def route_topk(h: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int):
+    """Routing by the largest logits: z = router h + bias (fp32, from h's stored values); the
+    `top` largest z win (ties: the lower index) and their weights are the softmax over the
+    winners' logits only.  Returns ids int32 [T, top] (by falling logit) and weights fp32
+    [T, top].  router fp32 [E, d], bias fp32 [E]."""
+    T = h.shape[0]
+    ids = torch.empty(T, top, dtype=torch.int32, device=h.device)
+    w = torch.empty(T, top, dtype=torch.float32, device=h.device)
+    if _native(h):
+        torch.ops.akap_stream.route_topk(ids, w, h, router, bias)
+        return ids, w
+    z = h.float() @ router.float().T
+    if bias is not None:
+        z = z + bias.float()
+    val, idx = z.topk(top, dim=-1)
+    ids.copy_(idx)
+    w.copy_(torch.softmax(val, dim=-1))
+    return ids, w
+
+
+def swiglu(gu: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t, f] = silu(gu[t, f]) gu[t, F + f] for gu [T, 2 F] = [gate | up] (fp32 arithmetic);
+    both may be column slices of wider rows."""
+    if _native(gu):
+        torch.ops.akap_stream.swiglu_routed(out, gu, None, None, 1)
+        return
+    F_ = gu.shape[1] // 2
+    out.copy_((torch.nn.functional.silu(gu[:, :F_].float()) * gu[:, F_:].float()).to(out.dtype))
+
+
+def swiglu_routed(gu: torch.Tensor, ids: torch.Tensor, w: torch.Tensor, experts: int,
+                  out: torch.Tensor) -> None:
+    """out[t, e F + f] = w_e(t) silu(gu[t, e 2F + f]) gu[t, e 2F + F + f], with w_e(t) the
+    routing weight of expert e for token t (0 when it was not chosen): the gated activation of
+    EVERY expert's [gate | up] projection, scaled so that one GEMM with the side-by-side
+    down-projections [d, E F] sums the chosen experts (small batches, where all expert weights
+    are streamed anyway)."""
+    if _native(gu):
+        torch.ops.akap_stream.swiglu_routed(out, gu, ids, w, int(experts))
+        return
+    T = gu.shape[0]
+    F_ = gu.shape[1] // (2 * experts)
+    full = torch.zeros(T, experts, dtype=torch.float32)
+    full.scatter_(1, ids.long(), w)
+    g3 = gu.float().view(T, experts, 2, F_)
+    act = torch.nn.functional.silu(g3[:, :, 0]) * g3[:, :, 1] * full[:, :, None]
+    out.copy_(act.view(T, experts * F_).to(out.dtype))
