@@ -1,0 +1,647 @@
+// Kernels of layers with a norm before and after each sublayer, decayed linear attention
+// ("retention") with a recurrent state, softmax attention whose heads mix their weights, and
+// logit-top-k routed gated experts.
+//
+// Sums of squares, norm scales, angles and rotations, decays, the recurrent state, attention
+// scores / softmax / head mixing / gates, router logits and the residual sum are fp32 whatever
+// the storage type; every size is a run-time argument.
+#include "../kernels/common.h"
+#include "stream.h"
+
+namespace akap_stream {
+
+using akap::bf16;
+using akap::block_sum;
+using akap::wave_max;
+using akap::wave_sum;
+
+namespace {
+
+template <typename T>
+__device__ __forceinline__ float ldf(const T* p) { return (float)*p; }
+template <typename T>
+__device__ __forceinline__ void stf(T* p, float v) { *p = (T)v; }
+
+__device__ __forceinline__ float sigmoidf(float z) { return 1.0f / (1.0f + __expf(-z)); }
+
+// ------------------------------------------------------------------ post-norm + residual + norm
+// one workgroup per row; a thread keeps to its own columns in every phase, so the two LDS rows
+// need no barrier beyond those of the block sums
+template <typename TY, typename TO>
+__global__ __launch_bounds__(256) void post_norm_add_norm_kernel(
+    TO* __restrict__ out, int out_stride, float* __restrict__ x, const TY* __restrict__ ya,
+    int ya_stride, const TY* __restrict__ yb, int yb_stride, const float* __restrict__ wa, int was,
+    const float* __restrict__ wb, int wbs, const float* __restrict__ post_w, int pws,
+    const float* __restrict__ next_w, int nws, int d, float eps, int fresh) {
+  extern __shared__ float lds[];
+  __shared__ float scratch[16];
+  float* ra = lds;
+  float* rb = lds + d;
+  const int row = blockIdx.x;
+  const TY* a = ya + (size_t)row * ya_stride;
+  const TY* b = yb ? yb + (size_t)row * yb_stride : nullptr;
+  float* xr = x + (size_t)row * d;
+  TO* o = out + (size_t)row * out_stride;
+  const float inv_d = 1.0f / (float)d;
+  float ss = 0.f, sb = 0.f;
+  for (int c = threadIdx.x; c < d; c += 256) {
+    const float f = ldf(a + c);
+    ra[c] = f;
+    ss += f * f;
+    if (b) {
+      const float g = ldf(b + c);
+      rb[c] = g;
+      sb += g * g;
+    }
+  }
+  ss = block_sum(ss, scratch);
+  if (b) {
+    sb = block_sum(sb, scratch);
+    const float ia = 1.0f / sqrtf(ss * inv_d + eps), ib = 1.0f / sqrtf(sb * inv_d + eps);
+    ss = 0.f;
+    for (int c = threadIdx.x; c < d; c += 256) {
+      const float m = 0.5f * (ra[c] * ia * wa[c * was] + rb[c] * ib * wb[c * wbs]);
+      ra[c] = m;
+      ss += m * m;
+    }
+    ss = block_sum(ss, scratch);
+  }
+  const float im = 1.0f / sqrtf(ss * inv_d + eps);
+  float sx = 0.f;
+  for (int c = threadIdx.x; c < d; c += 256) {
+    const float f = (fresh ? 0.f : xr[c]) + ra[c] * im * post_w[c * pws];
+    xr[c] = f;
+    ra[c] = f;
+    sx += f * f;
+  }
+  sx = block_sum(sx, scratch);
+  const float ix = 1.0f / sqrtf(sx * inv_d + eps);
+  for (int c = threadIdx.x; c < d; c += 256) stf(o + c, ra[c] * ix * next_w[c * nws]);
+}
+
+// ------------------------------------------------------------------ per-head norms + cache write
+// one workgroup per token; a wave per head (query heads, then key heads, then value heads)
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_cache_kernel(HeadNormParams p) {
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const T* row = (const T*)p.proj + (size_t)t * p.proj_stride;
+  const int64_t slot = p.slots[t];
+  const bool cached = slot >= 0 && slot < p.num_slots;
+  const int64_t blk = cached ? slot / p.BS : 0;
+  const int off = cached ? (int)(slot % p.BS) : 0;
+  for (int u = wave; u < p.H + 2 * p.G; u += 4) {
+    const T* src;
+    T* dst;
+    int n;
+    bool norm;
+    if (u < p.H) {
+      src = row + p.q_off + u * p.D;
+      dst = (T*)p.q_out + ((size_t)t * p.H + u) * p.D;
+      n = p.D;
+      norm = p.norm_qk;
+    } else if (u < p.H + p.G) {
+      if (!cached) continue;
+      const int g = u - p.H;
+      src = row + p.k_off + g * p.D;
+      dst = (T*)p.k_cache + ((size_t)(blk * p.G + g) * p.BS + off) * p.D;
+      n = p.D;
+      norm = p.norm_qk;
+    } else {
+      if (!cached) continue;
+      const int g = u - p.H - p.G;
+      src = row + p.v_off + g * p.Dv;
+      dst = (T*)p.v_cache + ((size_t)(blk * p.G + g) * p.BS + off) * p.Dv;
+      n = p.Dv;
+      norm = p.norm_v;
+    }
+    float inv = 1.0f;
+    if (norm) {
+      float ss = 0.f;
+      for (int c = lane; c < n; c += 64) {
+        const float f = ldf(src + c);
+        ss += f * f;
+      }
+      ss = wave_sum(ss);
+      inv = 1.0f / sqrtf(ss / (float)n + p.eps);
+    }
+    for (int c = lane; c < n; c += 64) stf(dst + c, ldf(src + c) * inv);
+  }
+}
+
+// ------------------------------------------------------------------ retention
+// One workgroup per (sequence, head).  A thread owns DREG consecutive state rows d of one
+// state column v: the state S[d][v] stays in registers over the sequence's rows of this step.
+// Rows are staged TC at a time: q and k rotated (fp32) into LDS, then the recurrence runs over
+// the TC tokens without a barrier (the DP lanes that share a column add their partial outputs
+// by lane exchange), then the outputs of the TC tokens are normed and gated, a wave per token.
+constexpr int RET_TC = 16;   // tokens staged at a time (8 when the rows of 16 exceed 64 KB)
+
+template <typename T, int DREG>
+__global__ __launch_bounds__(1024) void retention_kernel(RetentionParams p) {
+  extern __shared__ float lds[];
+  const int DP = p.DP;                    // lanes per column (power of two, <= 64)
+  const int DS = DREG + 4;                // padded part stride of the staged q / k rows
+  const int QS = DP * DS;
+  const int TC = p.TC;
+  float* qs = lds;                        // [TC][DP][DS]
+  float* ks = qs + TC * QS;
+  float* vs = ks + TC * QS;               // [TC][V]
+  float* os = vs + TC * p.V;              // [TC][V]
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int r0 = p.q_start ? p.q_start[b] : b;
+  const int r1 = p.q_start ? p.q_start[b + 1] : b + 1;
+  if (r1 <= r0) return;
+  const int slot = p.seq_slot[r0];
+  if (slot < 0 || slot >= p.num_slots) return;
+  const int tid = threadIdx.x, nt = blockDim.x;
+  const int v = tid / DP, part = tid % DP;
+  const bool owner = v < p.V;
+  const int d0 = part * DREG;
+  float* sp = p.state + (((size_t)slot * p.H + h) * p.V + (owner ? v : 0)) * p.D + d0;
+  float S[DREG];
+  const bool fresh = p.positions[r0] == 0;
+#pragma unroll
+  for (int i = 0; i < DREG; ++i) S[i] = (!fresh && owner && d0 + i < p.D) ? sp[i] : 0.f;
+  const float decay = exp2f(p.log2_decay[h]);
+  const float kscale = 1.0f / sqrtf((float)p.D);
+  const int half = p.rot_dims / 2;
+  const int wave = tid >> 6, lane = tid & 63, nw = nt >> 6;
+  for (int c0 = r0; c0 < r1; c0 += TC) {
+    const int n = min(TC, r1 - c0);
+    // stage: q, k (rotated, k scaled) and v of this head
+    const int DPD = DP * DREG;                // D rounded up to whole parts: the rest is zeros
+    for (int e = tid; e < n * DPD; e += nt) {
+      const int tk = e / DPD, d = e % DPD;
+      const T* row = (const T*)p.proj + (size_t)(c0 + tk) * p.proj_stride;
+      const T* q = row + p.q_off + h * p.D;
+      const T* k = row + p.k_off + h * p.D;
+      float qv = 0.f, kv = 0.f;
+      if (d < p.D) {
+        qv = ldf(q + d);
+        kv = ldf(k + d);
+      }
+      if (d < p.rot_dims) {
+        const int64_t pos = p.positions[c0 + tk];
+        const float* cs = p.cos_sin + (size_t)pos * p.rot_dims;
+        const int i = d < half ? d : d - half;
+        const float c = cs[i], s = cs[half + i];
+        if (d < half) {
+          const float q2 = ldf(q + d + half), k2 = ldf(k + d + half);
+          qv = qv * c - q2 * s;
+          kv = kv * c - k2 * s;
+        } else {
+          const float q1 = ldf(q + d - half), k1 = ldf(k + d - half);
+          qv = qv * c + q1 * s;
+          kv = kv * c + k1 * s;
+        }
+      }
+      const int o = tk * QS + (d / DREG) * DS + (d % DREG);
+      qs[o] = qv;
+      ks[o] = kv * kscale;
+    }
+    for (int e = tid; e < n * p.V; e += nt) {
+      const int tk = e / p.V, c = e % p.V;
+      vs[tk * p.V + c] =
+          ldf((const T*)p.proj + (size_t)(c0 + tk) * p.proj_stride + p.v_off + h * p.V + c);
+    }
+    __syncthreads();
+    // the recurrence
+    for (int tk = 0; tk < n; ++tk) {
+      const float vv = owner ? vs[tk * p.V + v] : 0.f;
+      const float* kq = ks + tk * QS + part * DS;
+      const float* qq = qs + tk * QS + part * DS;
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < DREG; i += 4) {
+        const float4 k4 = *(const float4*)(kq + i);
+        const float4 q4 = *(const float4*)(qq + i);
+        S[i] = fmaf(decay, S[i], k4.x * vv);
+        S[i + 1] = fmaf(decay, S[i + 1], k4.y * vv);
+        S[i + 2] = fmaf(decay, S[i + 2], k4.z * vv);
+        S[i + 3] = fmaf(decay, S[i + 3], k4.w * vv);
+        acc = fmaf(S[i], q4.x, acc);
+        acc = fmaf(S[i + 1], q4.y, acc);
+        acc = fmaf(S[i + 2], q4.z, acc);
+        acc = fmaf(S[i + 3], q4.w, acc);
+      }
+      for (int o = DP >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+      if (owner && part == 0) os[tk * p.V + v] = acc;
+    }
+    __syncthreads();
+    // output norm over the head's V entries and the silu gate
+    for (int tk = wave; tk < n; tk += nw) {
+      float ss = 0.f;
+      for (int c = lane; c < p.V; c += 64) {
+        const float f = os[tk * p.V + c];
+        ss += f * f;
+      }
+      ss = wave_sum(ss);
+      const float inv = 1.0f / sqrtf(ss / (float)p.V + p.eps);
+      const T* g = (const T*)p.proj + (size_t)(c0 + tk) * p.proj_stride + p.g_off + h * p.V;
+      T* o = (T*)p.out + (size_t)(c0 + tk) * p.out_stride + h * p.V;
+      for (int c = lane; c < p.V; c += 64) {
+        const float z = ldf(g + c);
+        stf(o + c, os[tk * p.V + c] * inv * z * sigmoidf(z));
+      }
+    }
+    __syncthreads();
+  }
+  if (owner) {
+#pragma unroll
+    for (int i = 0; i < DREG; ++i)
+      if (d0 + i < p.D) sp[i] = S[i];
+  }
+}
+
+// ------------------------------------------------------------------ head-mixed attention
+// One workgroup per (query row, key partition); thread (c, dv) owns entry dv of value head c and
+// keeps, for EVERY query head g, the unnormalised sum over the keys of exp(s_g - m_g) v_c[dv].
+// Keys go by pieces of 64: the waves score the piece (a lane per key, a wave per key head and
+// its query heads), publish the weights through LDS, then all threads accumulate.
+constexpr int TA_PIECE = 64;
+
+__device__ __forceinline__ int find_seq(const int32_t* q_start, int B, int t) {
+  int lo = 0, hi = B - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (q_start[mid] <= t) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+// the finish shared by the one-partition kernel and the merge: normalise, mix the heads, gate
+template <typename T, int HMAX>
+__device__ __forceinline__ void talk_finish(const TalkParams& p, int t, int c, int dv,
+                                            float (&acc)[HMAX], const float* inv_l) {
+  const int rep = p.H / p.G;
+#pragma unroll
+  for (int g = 0; g < HMAX; ++g)
+    if (g < p.H) acc[g] *= inv_l[g];
+  for (int i = 0; i < rep; ++i) {
+    const int h = c * rep + i;
+    float o;
+    if (p.talk) {
+      o = 0.f;
+      const float* tr = p.talk + (size_t)h * p.H;
+#pragma unroll
+      for (int g = 0; g < HMAX; ++g)
+        if (g < p.H) o = fmaf(tr[g], acc[g], o);
+    } else {
+      o = 0.f;
+#pragma unroll
+      for (int g = 0; g < HMAX; ++g)
+        if (g == h) o = acc[g];
+    }
+    const int col = h * p.Dv + dv;
+    if (p.gate) o *= sigmoidf(ldf((const T*)p.gate + (size_t)t * p.gate_stride + col));
+    stf((T*)p.out + (size_t)t * p.out_stride + col, o);
+  }
+}
+
+template <typename T, int HMAX>
+__global__ __launch_bounds__(1024) void talking_attention_kernel(TalkParams p) {
+  extern __shared__ float lds[];
+  float* qs = lds;                                 // [H][D]
+  float* ps = qs + p.H * p.D;                      // [H][PIECE] weights of the piece
+  float* alpha = ps + p.H * TA_PIECE;              // [H] rescale of the running sums
+  float* ms = alpha + p.H;                         // [H] running max
+  float* lsum = ms + p.H;                          // [H] running sum
+  int* rowbase = (int*)(lsum + p.H);               // [PIECE] cache row of key j for head 0
+  const int t = blockIdx.x, part = blockIdx.y;
+  const int b = p.q_start ? find_seq(p.q_start, p.B, t) : t;
+  if (p.seq_lens[b] <= 0) return;
+  const int tid = threadIdx.x, nt = blockDim.x;
+  const int wave = tid >> 6, lane = tid & 63, nw = nt >> 6;
+  const int nkeys = (int)p.positions[t] + 1;
+  const int pieces = (nkeys + TA_PIECE - 1) / TA_PIECE;
+  const int per = (pieces + p.num_parts - 1) / p.num_parts;
+  const int lo = part * per * TA_PIECE;
+  const int hi = min(nkeys, lo + per * TA_PIECE);
+  const int rep = p.H / p.G;
+  const int GV = p.G * p.Dv;
+  const bool owner = tid < GV;
+  const int c = owner ? tid / p.Dv : 0, dv = owner ? tid % p.Dv : 0;
+  float acc[HMAX];
+#pragma unroll
+  for (int g = 0; g < HMAX; ++g) acc[g] = 0.f;
+  for (int e = tid; e < p.H * p.D; e += nt) qs[e] = ldf((const T*)p.q + (size_t)t * p.H * p.D + e);
+  for (int g = tid; g < p.H; g += nt) { ms[g] = -INFINITY; lsum[g] = 0.f; }
+  __syncthreads();
+  const int32_t* bt = p.block_tables + (size_t)b * p.max_blocks;
+  for (int j0 = lo; j0 < hi; j0 += TA_PIECE) {
+    const int j = j0 + lane;
+    const bool live = j < hi;
+    int base = 0;
+    if (live) base = (bt[j / p.BS] * p.G) * p.BS + (j % p.BS);
+    if (wave == 0) rowbase[lane] = base;
+    // scores: wave w takes key heads w, w + nw, ...; lane = key
+    for (int kc = wave; kc < p.G; kc += nw) {
+      const T* kr = (const T*)p.k_cache + (size_t)(base + kc * p.BS) * p.D;
+      for (int i0 = 0; i0 < rep; i0 += 4) {
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        const float* q0 = qs + (kc * rep + i0) * p.D;
+        const int n = min(4, rep - i0);
+        if (live) {
+          for (int d = 0; d < p.D; ++d) {
+            const float kv = ldf(kr + d);
+            s0 = fmaf(q0[d], kv, s0);
+            if (n > 1) s1 = fmaf(q0[p.D + d], kv, s1);
+            if (n > 2) s2 = fmaf(q0[2 * p.D + d], kv, s2);
+            if (n > 3) s3 = fmaf(q0[3 * p.D + d], kv, s3);
+          }
+        }
+        const float sc[4] = {s0, s1, s2, s3};
+        for (int i = 0; i < n; ++i) {
+          const int g = kc * rep + i0 + i;
+          const float s = live ? sc[i] * p.scale : -INFINITY;
+          const float m_old = ms[g];
+          const float m_new = fmaxf(m_old, wave_max(s));
+          const float pw = live ? __expf(s - m_new) : 0.f;
+          const float sum = wave_sum(pw);
+          ps[g * TA_PIECE + lane] = pw;
+          if (lane == 0) {
+            const float a = m_old == -INFINITY ? 0.f : __expf(m_old - m_new);
+            alpha[g] = a;
+            ms[g] = m_new;
+            lsum[g] = lsum[g] * a + sum;
+          }
+        }
+      }
+    }
+    __syncthreads();
+    if (owner) {
+#pragma unroll
+      for (int g = 0; g < HMAX; ++g)
+        if (g < p.H) acc[g] *= alpha[g];
+      const int nk = min(TA_PIECE, hi - j0);
+      const T* vb = (const T*)p.v_cache + (size_t)c * p.BS * p.Dv + dv;
+      int jj = 0;
+      for (; jj + 4 <= nk; jj += 4) {
+        const float v0 = ldf(vb + (size_t)rowbase[jj] * p.Dv);
+        const float v1 = ldf(vb + (size_t)rowbase[jj + 1] * p.Dv);
+        const float v2 = ldf(vb + (size_t)rowbase[jj + 2] * p.Dv);
+        const float v3 = ldf(vb + (size_t)rowbase[jj + 3] * p.Dv);
+#pragma unroll
+        for (int g = 0; g < HMAX; ++g) {
+          if (g < p.H) {
+            const float4 w4 = *(const float4*)(ps + g * TA_PIECE + jj);
+            acc[g] = fmaf(w4.x, v0, acc[g]);
+            acc[g] = fmaf(w4.y, v1, acc[g]);
+            acc[g] = fmaf(w4.z, v2, acc[g]);
+            acc[g] = fmaf(w4.w, v3, acc[g]);
+          }
+        }
+      }
+      for (; jj < nk; ++jj) {
+        const float v0 = ldf(vb + (size_t)rowbase[jj] * p.Dv);
+#pragma unroll
+        for (int g = 0; g < HMAX; ++g)
+          if (g < p.H) acc[g] = fmaf(ps[g * TA_PIECE + jj], v0, acc[g]);
+      }
+    }
+    __syncthreads();
+  }
+  if (p.num_parts == 1) {
+    // 1 / l per head (lsum > 0: key 0 is always visible)
+    for (int g = tid; g < p.H; g += nt) alpha[g] = 1.0f / lsum[g];
+    __syncthreads();
+    if (owner) talk_finish<T, HMAX>(p, t, c, dv, acc, alpha);
+    return;
+  }
+  const size_t cell = (size_t)t * p.num_parts + part;
+  for (int g = tid; g < p.H; g += nt) {
+    p.ws_ml[(cell * p.H + g) * 2] = ms[g];
+    p.ws_ml[(cell * p.H + g) * 2 + 1] = lsum[g];
+  }
+  if (owner) {
+#pragma unroll
+    for (int g = 0; g < HMAX; ++g)
+      if (g < p.H) p.ws_o[(cell * p.H + g) * GV + tid] = acc[g];
+  }
+}
+
+template <typename T, int HMAX>
+__global__ __launch_bounds__(1024) void talking_merge_kernel(TalkParams p) {
+  extern __shared__ float lds[];
+  float* wgt = lds;                  // [parts][H] weight of a partition's sums
+  float* inv_l = wgt + p.num_parts * p.H;
+  const int t = blockIdx.x;
+  const int b = p.q_start ? find_seq(p.q_start, p.B, t) : t;
+  if (p.seq_lens[b] <= 0) return;
+  const int tid = threadIdx.x, nt = blockDim.x;
+  const int GV = p.G * p.Dv;
+  for (int g = tid; g < p.H; g += nt) {
+    float mx = -INFINITY;
+    for (int q = 0; q < p.num_parts; ++q)
+      mx = fmaxf(mx, p.ws_ml[(((size_t)t * p.num_parts + q) * p.H + g) * 2]);
+    float tot = 0.f;
+    for (int q = 0; q < p.num_parts; ++q) {
+      const float* ml = p.ws_ml + (((size_t)t * p.num_parts + q) * p.H + g) * 2;
+      const float w = ml[0] == -INFINITY ? 0.f : __expf(ml[0] - mx);
+      wgt[q * p.H + g] = w;
+      tot += ml[1] * w;
+    }
+    inv_l[g] = 1.0f / tot;
+  }
+  __syncthreads();
+  if (tid >= GV) return;
+  float acc[HMAX];
+#pragma unroll
+  for (int g = 0; g < HMAX; ++g) acc[g] = 0.f;
+  for (int q = 0; q < p.num_parts; ++q) {
+    const float* o = p.ws_o + ((size_t)t * p.num_parts + q) * p.H * GV + tid;
+#pragma unroll
+    for (int g = 0; g < HMAX; ++g)
+      if (g < p.H) {
+        const float w = wgt[q * p.H + g];
+        if (w != 0.f) acc[g] = fmaf(w, o[(size_t)g * GV], acc[g]);
+      }
+  }
+  talk_finish<T, HMAX>(p, t, tid / p.Dv, tid % p.Dv, acc, inv_l);
+}
+
+// ------------------------------------------------------------------ routing by the largest logits
+template <typename T>
+__global__ __launch_bounds__(256) void route_topk_kernel(int32_t* __restrict__ ids,
+                                                         float* __restrict__ wout,
+                                                         const T* __restrict__ h, int h_stride,
+                                                         const float* __restrict__ router,
+                                                         const float* __restrict__ bias, int d,
+                                                         int n, int top) {
+  extern __shared__ float lds[];   // [n] logits
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const T* hr = h + (size_t)t * h_stride;
+  for (int e = wave; e < n; e += 4) {
+    const float* wr = router + (size_t)e * d;
+    float a = 0.f;
+    for (int c = lane; c < d; c += 64) a = fmaf(ldf(hr + c), wr[c], a);
+    a = wave_sum(a);
+    if (lane == 0) lds[e] = a + (bias ? bias[e] : 0.f);
+  }
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  float first = 0.f, total = 0.f;
+  for (int k = 0; k < top; ++k) {
+    int best = -1;
+    float bv = 0.f;
+    for (int e = 0; e < n; ++e) {
+      const float v = lds[e];
+      if (v != v || v == -INFINITY) continue;     // taken (marked below) or unusable
+      if (best < 0 || v > bv) { best = e; bv = v; }
+    }
+    if (best < 0) best = 0;
+    lds[best] = -INFINITY;
+    if (k == 0) first = bv;
+    const float ev = __expf(bv - first);
+    ids[(size_t)t * top + k] = best;
+    wout[(size_t)t * top + k] = ev;
+    total += ev;
+  }
+  const float inv = 1.0f / total;
+  for (int k = 0; k < top; ++k) wout[(size_t)t * top + k] *= inv;
+}
+
+// out[t, e F + f] = w_e(t) silu(gu[t, e 2F + f]) gu[t, e 2F + F + f]; ids null: weight 1
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_routed_kernel(T* __restrict__ out, int out_stride,
+                                                            const T* __restrict__ gu, int gu_stride,
+                                                            const int32_t* __restrict__ ids,
+                                                            const float* __restrict__ w, int top,
+                                                            int E, int F) {
+  extern __shared__ float lds[];   // [E] routing weight of every expert
+  const int t = blockIdx.x;
+  for (int e = threadIdx.x; e < E; e += 256) lds[e] = ids ? 0.f : 1.f;
+  __syncthreads();
+  if (ids && threadIdx.x < top) {
+    const int e = ids[(size_t)t * top + threadIdx.x];
+    if (e >= 0 && e < E) lds[e] = w[(size_t)t * top + threadIdx.x];
+  }
+  __syncthreads();
+  const T* g = gu + (size_t)t * gu_stride;
+  T* o = out + (size_t)t * out_stride;
+  for (int c = threadIdx.x; c < E * F; c += 256) {
+    const int e = c / F, f = c - e * F;
+    const float we = lds[e];
+    float r = 0.f;
+    if (we != 0.f) {
+      const float z = ldf(g + e * 2 * F + f);
+      r = we * z * sigmoidf(z) * ldf(g + e * 2 * F + F + f);
+    }
+    stf(o + c, r);
+  }
+}
+
+}  // namespace
+
+// ================================================================== launchers
+void launch_post_norm_add_norm(void* out, bool out_f32, int out_stride, float* x, const void* ya,
+                               int ya_stride, const void* yb, int yb_stride, bool y_f32,
+                               const float* wa, int was, const float* wb, int wbs,
+                               const float* post_w, int pws, const float* next_w, int nws,
+                               int rows, int d, float eps, bool fresh, hipStream_t s) {
+  if (rows <= 0) return;
+  const size_t lds = (size_t)2 * d * sizeof(float);
+#define AKAP_PN(TY, TO)                                                                         \
+  post_norm_add_norm_kernel<TY, TO><<<rows, 256, lds, s>>>(                                     \
+      (TO*)out, out_stride, x, (const TY*)ya, ya_stride, (const TY*)yb, yb_stride, wa, was, wb, \
+      wbs, post_w, pws, next_w, nws, d, eps, fresh ? 1 : 0)
+  if (y_f32 && out_f32) AKAP_PN(float, float);
+  else if (y_f32) AKAP_PN(float, bf16);
+  else if (out_f32) AKAP_PN(bf16, float);
+  else AKAP_PN(bf16, bf16);
+#undef AKAP_PN
+}
+
+void launch_head_norm_cache(const HeadNormParams& p, bool f32, hipStream_t s) {
+  if (p.T <= 0) return;
+  if (f32) head_norm_cache_kernel<float><<<p.T, 256, 0, s>>>(p);
+  else head_norm_cache_kernel<bf16><<<p.T, 256, 0, s>>>(p);
+}
+
+int retention_dreg(int D, int V) {
+  // state rows per thread: the fewest of 16 / 32 / 64 that keeps the workgroup within 1024
+  // threads (V columns x D / DREG lanes each, the lanes of a column a power of two)
+  for (int dreg : {16, 32, 64}) {
+    int dp = 1;
+    while (dp * dreg < D) dp <<= 1;
+    if (dp <= 64 && (int64_t)V * dp <= 1024) return dreg;
+  }
+  return 0;
+}
+
+void launch_retention(RetentionParams p, bool f32, hipStream_t s) {
+  if (p.num_seqs <= 0) return;
+  const int dreg = retention_dreg(p.D, p.V);
+  int dp = 1;
+  while (dp * dreg < p.D) dp <<= 1;
+  p.DP = dp;
+  const int nt = ((p.V * dp + 63) / 64) * 64;
+  p.TC = RET_TC;
+  size_t lds = (size_t)p.TC * (2 * dp * (dreg + 4) + 2 * p.V) * sizeof(float);
+  if (lds > 65536) {
+    p.TC = RET_TC / 2;
+    lds /= 2;
+  }
+  const dim3 grid(p.num_seqs, p.H);
+#define AKAP_RET(TY, R) retention_kernel<TY, R><<<grid, nt, lds, s>>>(p)
+  if (f32) {
+    if (dreg == 16) AKAP_RET(float, 16); else if (dreg == 32) AKAP_RET(float, 32); else AKAP_RET(float, 64);
+  } else {
+    if (dreg == 16) AKAP_RET(bf16, 16); else if (dreg == 32) AKAP_RET(bf16, 32); else AKAP_RET(bf16, 64);
+  }
+#undef AKAP_RET
+}
+
+size_t talking_attention_lds(int H, int D) {
+  return (size_t)(H * D + H * TA_PIECE + 3 * H + TA_PIECE) * sizeof(float);
+}
+
+void launch_talking_attention(const TalkParams& p, bool f32, hipStream_t s) {
+  if (p.T <= 0) return;
+  const int nt = ((p.G * p.Dv + 63) / 64) * 64;
+  const size_t lds = talking_attention_lds(p.H, p.D);
+  const int rows = p.T;
+  const dim3 grid(rows, p.num_parts);
+  const size_t mlds = (size_t)(p.num_parts + 1) * p.H * sizeof(float);
+#define AKAP_TA(TY, HM)                                                          \
+  do {                                                                           \
+    talking_attention_kernel<TY, HM><<<grid, nt, lds, s>>>(p);                   \
+    if (p.num_parts > 1) talking_merge_kernel<TY, HM><<<rows, nt, mlds, s>>>(p); \
+  } while (0)
+  if (f32) {
+    if (p.H <= 8) AKAP_TA(float, 8); else if (p.H <= 16) AKAP_TA(float, 16); else AKAP_TA(float, 32);
+  } else {
+    if (p.H <= 8) AKAP_TA(bf16, 8); else if (p.H <= 16) AKAP_TA(bf16, 16); else AKAP_TA(bf16, 32);
+  }
+#undef AKAP_TA
+}
+
+void launch_route_topk(int32_t* ids, float* w, const void* h, int h_stride, const float* router,
+                       const float* bias, int rows, int d, int n, int top, bool f32,
+                       hipStream_t s) {
+  if (rows <= 0) return;
+  const size_t lds = (size_t)n * sizeof(float);
+  if (f32)
+    route_topk_kernel<float><<<rows, 256, lds, s>>>(ids, w, (const float*)h, h_stride, router, bias,
+                                                    d, n, top);
+  else
+    route_topk_kernel<bf16><<<rows, 256, lds, s>>>(ids, w, (const bf16*)h, h_stride, router, bias,
+                                                   d, n, top);
+}
+
+void launch_swiglu_routed(void* out, int out_stride, const void* gu, int gu_stride,
+                          const int32_t* ids, const float* w, int rows, int top, int E, int F,
+                          bool f32, hipStream_t s) {
+  if (rows <= 0) return;
+  const size_t lds = (size_t)E * sizeof(float);
+  if (f32)
+    swiglu_routed_kernel<float><<<rows, 256, lds, s>>>((float*)out, out_stride, (const float*)gu,
+                                                       gu_stride, ids, w, top, E, F);
+  else
+    swiglu_routed_kernel<bf16><<<rows, 256, lds, s>>>((bf16*)out, out_stride, (const bf16*)gu,
+                                                      gu_stride, ids, w, top, E, F);
+}
+
+}  // namespace akap_stream

@@ -160,4 +160,82 @@ void launch_moe_combine(float* out, const void* y, const int32_t* inv, const int
                         const float* w, const void* h, int h_stride, int rows, int d, int top,
                         int E, int y_rows, bool f32, hipStream_t s);
 
+// ---- sandwich norms, retention, head-mixed attention, logit-top-k routing (retention.hip) -------
+// m = ya, or (rms(ya) wa + rms(yb) wb) / 2 when yb is given; x (fp32 rows of d) <- x + rms(m)
+// post_w (fresh: x is not read); out = rms(x) next_w.  Every weight has a stride of 1 (d
+// entries) or 0 (one number).  ya / yb are both fp32 or both of the activation type.
+void launch_post_norm_add_norm(void* out, bool out_f32, int out_stride, float* x, const void* ya,
+                               int ya_stride, const void* yb, int yb_stride, bool y_f32,
+                               const float* wa, int was, const float* wb, int wbs,
+                               const float* post_w, int pws, const float* next_w, int nws,
+                               int rows, int d, float eps, bool fresh, hipStream_t s);
+
+struct HeadNormParams {
+  const void* proj;   // [T, N] fused projection rows
+  int proj_stride;
+  void* q_out;        // [T, H, D]
+  void* k_cache;      // [NB, G, BS, D]
+  void* v_cache;      // [NB, G, BS, Dv]
+  const int64_t* slots;
+  int T, H, G, D, Dv, BS, q_off, k_off, v_off;
+  int64_t num_slots;  // NB * BS
+  float eps;
+  bool norm_qk, norm_v;
+};
+void launch_head_norm_cache(const HeadNormParams& p, bool f32, hipStream_t s);
+
+struct RetentionParams {
+  void* out;            // rows of out_stride elements; head h at columns [h V, (h + 1) V)
+  int out_stride;
+  const void* proj;     // [T, N] fused projection rows
+  int proj_stride;
+  int q_off, k_off, v_off, g_off;
+  float* state;         // [slots, H, V, D]: the transposed state of every slot and head
+  int num_slots;
+  const int32_t* seq_slot;   // [T]
+  const int64_t* positions;  // [T]
+  const int32_t* q_start;    // [num_seqs + 1] or null (row t is sequence t)
+  const float* cos_sin;      // [max_pos, rot_dims] = [cos | sin] or null
+  int rot_dims;
+  const float* log2_decay;   // [H]
+  int num_seqs, H, D, V;
+  float eps;
+  int DP, TC;           // set by the launcher
+};
+// 0 when the sizes do not fit a workgroup (V columns x ceil(D / 64) lanes > 1024 threads)
+int retention_dreg(int D, int V);
+void launch_retention(RetentionParams p, bool f32, hipStream_t s);
+
+struct TalkParams {
+  void* out;            // rows of out_stride elements; head h at columns [h Dv, (h + 1) Dv)
+  int out_stride;
+  const void* q;        // [T, H, D]
+  const void* k_cache;  // [NB, G, BS, D]
+  const void* v_cache;  // [NB, G, BS, Dv]
+  const int32_t* block_tables;  // [B, max_blocks]
+  int max_blocks;
+  const int32_t* seq_lens;      // [B]
+  const int32_t* q_start;       // [B + 1] or null (row t is sequence t)
+  const int64_t* positions;     // [T]
+  const float* talk;    // [H, H] or null
+  const void* gate;     // [T, H Dv] logits with row stride gate_stride, or null
+  int gate_stride;
+  float scale;
+  int T, B, H, G, D, Dv, BS;
+  // split form: (max, sum) [T, parts, H, 2] and unnormalised sums [T, parts, H, G Dv]
+  float* ws_ml;
+  float* ws_o;
+  int num_parts;
+};
+size_t talking_attention_lds(int H, int D);
+void launch_talking_attention(const TalkParams& p, bool f32, hipStream_t s);
+
+void launch_route_topk(int32_t* ids, float* w, const void* h, int h_stride, const float* router,
+                       const float* bias, int rows, int d, int n, int top, bool f32,
+                       hipStream_t s);
+// ids null: every weight is 1 (E = 1: a plain gated activation of [gate | up] rows)
+void launch_swiglu_routed(void* out, int out_stride, const void* gu, int gu_stride,
+                          const int32_t* ids, const float* w, int rows, int top, int E, int F,
+                          bool f32, hipStream_t s);
+
 }  // namespace akap_stream

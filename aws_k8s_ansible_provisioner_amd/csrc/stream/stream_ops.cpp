@@ -684,6 +684,248 @@ void moe_combine(Tensor out, Tensor y, std::optional<Tensor> inv, Tensor ids, Te
                                   is_f32(y, "y"), cur_stream());
 }
 
+// a norm weight: fp32 with d entries (stride 1) or one (stride 0)
+int weight_stride(const Tensor& w, int64_t d, const char* name) {
+  TORCH_CHECK(w.is_cuda() && w.scalar_type() == at::kFloat && w.is_contiguous() &&
+                  (w.numel() == d || w.numel() == 1), name, " must be fp32 with d entries or one");
+  return w.numel() == 1 ? 0 : 1;
+}
+
+void post_norm_add_norm(Tensor out, Tensor x, Tensor ya, std::optional<Tensor> yb,
+                        std::optional<Tensor> wa, std::optional<Tensor> wb, Tensor post_w,
+                        Tensor next_w, double eps, bool fresh) {
+  CHECK_GPU(out); CHECK_GPU(x); CHECK_GPU(ya);
+  CHECK_F32(x); CHECK_CONTIG(x); CHECK_LAST_CONTIG(out); CHECK_LAST_CONTIG(ya);
+  TORCH_CHECK(x.dim() == 2 && out.dim() == 2 && out.sizes() == x.sizes() && ya.dim() == 2 &&
+                  ya.sizes() == x.sizes(), "post_norm_add_norm: shapes");
+  const int64_t rows = x.size(0), d = x.size(1);
+  TORCH_CHECK(d * 8 <= 65536, "post_norm_add_norm: rows of at most 8192 entries");
+  const bool yf = is_f32(ya, "ya");
+  const void* ybp = nullptr;
+  const float *wap = nullptr, *wbp = nullptr;
+  int ybs = 0, was = 0, wbs = 0;
+  if (yb.has_value()) {
+    CHECK_GPU(*yb); CHECK_LAST_CONTIG(*yb);
+    TORCH_CHECK(yb->sizes() == x.sizes() && yb->scalar_type() == ya.scalar_type() &&
+                    wa.has_value() && wb.has_value(),
+                "post_norm_add_norm: two branches need yb of ya's shape and type, wa and wb");
+    ybp = yb->data_ptr();
+    ybs = yb->stride(0);
+    was = weight_stride(*wa, d, "wa");
+    wbs = weight_stride(*wb, d, "wb");
+    wap = wa->data_ptr<float>();
+    wbp = wb->data_ptr<float>();
+  }
+  const int pws = weight_stride(post_w, d, "post_w"), nws = weight_stride(next_w, d, "next_w");
+  const c10::DeviceGuard g(x.device());
+  akap_stream::launch_post_norm_add_norm(
+      out.data_ptr(), is_f32(out, "out"), (int)out.stride(0), x.data_ptr<float>(), ya.data_ptr(),
+      (int)ya.stride(0), ybp, ybs, yf, wap, was, wbp, wbs, post_w.data_ptr<float>(), pws,
+      next_w.data_ptr<float>(), nws, (int)rows, (int)d, (float)eps, fresh, cur_stream());
+}
+
+void head_norm_cache(Tensor proj, Tensor q_out, Tensor k_cache, Tensor v_cache, Tensor slots,
+                     int64_t H, int64_t G, int64_t D, int64_t Dv, int64_t q_off, int64_t k_off,
+                     int64_t v_off, double eps, bool norm_qk, bool norm_v) {
+  CHECK_GPU(proj); CHECK_GPU(q_out); CHECK_GPU(k_cache); CHECK_GPU(v_cache); CHECK_GPU(slots);
+  CHECK_LAST_CONTIG(proj); CHECK_CONTIG(q_out); CHECK_CONTIG(k_cache); CHECK_CONTIG(v_cache);
+  CHECK_CONTIG(slots);
+  const bool f32 = is_f32(proj, "proj");
+  TORCH_CHECK(q_out.scalar_type() == proj.scalar_type() &&
+                  k_cache.scalar_type() == proj.scalar_type() &&
+                  v_cache.scalar_type() == proj.scalar_type(), "head_norm_cache: dtypes differ");
+  TORCH_CHECK(slots.scalar_type() == at::kLong, "slots must be int64");
+  const int64_t T = proj.size(0), N = proj.size(1);
+  TORCH_CHECK(proj.dim() == 2 && H > 0 && G > 0 && D > 0 && Dv > 0 && q_off >= 0 && k_off >= 0 &&
+                  v_off >= 0 && q_off + H * D <= N && k_off + G * D <= N && v_off + G * Dv <= N,
+              "head_norm_cache: slices outside the projection");
+  TORCH_CHECK(q_out.numel() == T * H * D && slots.numel() == T, "head_norm_cache: q_out / slots");
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.size(1) == G &&
+                  k_cache.size(3) == D && v_cache.size(0) == k_cache.size(0) &&
+                  v_cache.size(1) == G && v_cache.size(2) == k_cache.size(2) &&
+                  v_cache.size(3) == Dv, "head_norm_cache: cache shapes");
+  akap_stream::HeadNormParams p;
+  p.proj = proj.data_ptr(); p.proj_stride = proj.stride(0);
+  p.q_out = q_out.data_ptr(); p.k_cache = k_cache.data_ptr(); p.v_cache = v_cache.data_ptr();
+  p.slots = slots.data_ptr<int64_t>();
+  p.T = T; p.H = H; p.G = G; p.D = D; p.Dv = Dv; p.BS = k_cache.size(2);
+  p.q_off = q_off; p.k_off = k_off; p.v_off = v_off;
+  p.num_slots = k_cache.size(0) * k_cache.size(2);
+  p.eps = (float)eps; p.norm_qk = norm_qk; p.norm_v = norm_v;
+  const c10::DeviceGuard g(proj.device());
+  akap_stream::launch_head_norm_cache(p, f32, cur_stream());
+}
+
+void retention(Tensor out, Tensor proj, int64_t q_off, int64_t k_off, int64_t v_off, int64_t g_off,
+               Tensor state, Tensor seq_slot, Tensor positions, std::optional<Tensor> q_start,
+               std::optional<Tensor> cos_sin, Tensor log2_decay, int64_t H, int64_t D, int64_t V,
+               double eps) {
+  CHECK_GPU(out); CHECK_GPU(proj); CHECK_GPU(state); CHECK_GPU(seq_slot); CHECK_GPU(positions);
+  CHECK_GPU(log2_decay);
+  CHECK_LAST_CONTIG(out); CHECK_LAST_CONTIG(proj); CHECK_CONTIG(state); CHECK_F32(state);
+  CHECK_CONTIG(seq_slot); CHECK_CONTIG(positions); CHECK_CONTIG(log2_decay); CHECK_F32(log2_decay);
+  const bool f32 = is_f32(proj, "proj");
+  TORCH_CHECK(out.scalar_type() == proj.scalar_type(), "retention: dtypes differ");
+  TORCH_CHECK(seq_slot.scalar_type() == at::kInt && positions.scalar_type() == at::kLong,
+              "retention: seq_slot int32, positions int64");
+  const int64_t T = proj.size(0), N = proj.size(1);
+  TORCH_CHECK(proj.dim() == 2 && out.dim() == 2 && out.size(0) == T && out.size(1) >= H * V &&
+                  H > 0 && D > 0 && V > 0, "retention: shapes");
+  TORCH_CHECK(q_off >= 0 && k_off >= 0 && v_off >= 0 && g_off >= 0 && q_off + H * D <= N &&
+                  k_off + H * D <= N && v_off + H * V <= N && g_off + H * V <= N,
+              "retention: slices outside the projection");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == V && state.size(3) == D,
+              "retention: state must be [slots, H, V, D]");
+  TORCH_CHECK(seq_slot.numel() >= T && positions.numel() >= T && log2_decay.numel() == H,
+              "retention: seq_slot / positions / decay sizes");
+  TORCH_CHECK(akap_stream::retention_dreg((int)D, (int)V) > 0,
+              "retention: head sizes too large for one workgroup (V * ceil(D / 64) <= 1024)");
+  akap_stream::RetentionParams p;
+  p.out = out.data_ptr(); p.out_stride = out.stride(0);
+  p.proj = proj.data_ptr(); p.proj_stride = proj.stride(0);
+  p.q_off = q_off; p.k_off = k_off; p.v_off = v_off; p.g_off = g_off;
+  p.state = state.data_ptr<float>(); p.num_slots = state.size(0);
+  p.seq_slot = seq_slot.data_ptr<int32_t>(); p.positions = positions.data_ptr<int64_t>();
+  p.q_start = nullptr;
+  p.num_seqs = T;
+  if (q_start.has_value()) {
+    CHECK_GPU(*q_start); CHECK_CONTIG(*q_start);
+    TORCH_CHECK(q_start->scalar_type() == at::kInt && q_start->numel() >= 1, "retention: q_start");
+    p.q_start = q_start->data_ptr<int32_t>();
+    p.num_seqs = q_start->numel() - 1;
+  }
+  p.cos_sin = nullptr; p.rot_dims = 0;
+  if (cos_sin.has_value()) {
+    CHECK_GPU(*cos_sin); CHECK_CONTIG(*cos_sin); CHECK_F32(*cos_sin);
+    TORCH_CHECK(cos_sin->dim() == 2 && cos_sin->size(1) % 2 == 0 && cos_sin->size(1) <= D,
+                "retention: cos_sin must be [max_pos, dims <= D]");
+    p.cos_sin = cos_sin->data_ptr<float>();
+    p.rot_dims = cos_sin->size(1);
+  }
+  p.log2_decay = log2_decay.data_ptr<float>();
+  p.H = H; p.D = D; p.V = V; p.eps = (float)eps; p.DP = 1;
+  const c10::DeviceGuard g(proj.device());
+  akap_stream::launch_retention(p, f32, cur_stream());
+}
+
+void talking_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables,
+                       Tensor seq_lens, std::optional<Tensor> q_start, Tensor positions,
+                       std::optional<Tensor> talk, std::optional<Tensor> gate, double scale,
+                       std::optional<Tensor> ws_ml, std::optional<Tensor> ws_o, int64_t num_parts) {
+  CHECK_GPU(out); CHECK_GPU(q); CHECK_GPU(k_cache); CHECK_GPU(v_cache); CHECK_GPU(block_tables);
+  CHECK_GPU(seq_lens); CHECK_GPU(positions);
+  CHECK_LAST_CONTIG(out); CHECK_CONTIG(q); CHECK_CONTIG(k_cache); CHECK_CONTIG(v_cache);
+  CHECK_CONTIG(seq_lens); CHECK_CONTIG(positions);
+  const bool f32 = is_f32(q, "q");
+  TORCH_CHECK(out.scalar_type() == q.scalar_type() && k_cache.scalar_type() == q.scalar_type() &&
+                  v_cache.scalar_type() == q.scalar_type(), "talking_attention: dtypes differ");
+  TORCH_CHECK(q.dim() == 3 && k_cache.dim() == 4 && v_cache.dim() == 4, "talking_attention: ranks");
+  const int64_t T = q.size(0), H = q.size(1), D = q.size(2);
+  const int64_t G = k_cache.size(1), BS = k_cache.size(2), Dv = v_cache.size(3);
+  TORCH_CHECK(k_cache.size(3) == D && v_cache.size(0) == k_cache.size(0) && v_cache.size(1) == G &&
+                  v_cache.size(2) == BS && G > 0 && H % G == 0, "talking_attention: cache shapes");
+  TORCH_CHECK(H <= 32 && G * Dv <= 1024,
+              "talking_attention: at most 32 heads and 1024 value entries per token");
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) >= H * Dv, "talking_attention: out");
+  TORCH_CHECK(block_tables.dim() == 2 && block_tables.scalar_type() == at::kInt &&
+                  block_tables.stride(1) == 1 && seq_lens.scalar_type() == at::kInt &&
+                  positions.scalar_type() == at::kLong && positions.numel() >= T,
+              "talking_attention: block_tables / seq_lens int32, positions int64");
+  akap_stream::TalkParams p;
+  p.out = out.data_ptr(); p.out_stride = out.stride(0);
+  p.q = q.data_ptr(); p.k_cache = k_cache.data_ptr(); p.v_cache = v_cache.data_ptr();
+  TORCH_CHECK(block_tables.stride(0) == block_tables.size(1) || block_tables.size(0) == 1,
+              "talking_attention: block_tables rows must be dense");
+  p.block_tables = block_tables.data_ptr<int32_t>(); p.max_blocks = block_tables.size(1);
+  p.seq_lens = seq_lens.data_ptr<int32_t>();
+  p.B = seq_lens.numel();
+  TORCH_CHECK(block_tables.size(0) >= p.B, "talking_attention: a block-table row per sequence");
+  p.q_start = nullptr;
+  if (q_start.has_value()) {
+    CHECK_GPU(*q_start); CHECK_CONTIG(*q_start);
+    TORCH_CHECK(q_start->scalar_type() == at::kInt && q_start->numel() >= p.B + 1,
+                "talking_attention: q_start");
+    p.q_start = q_start->data_ptr<int32_t>();
+  } else {
+    TORCH_CHECK(p.B >= T, "talking_attention: a sequence per row when q_start is not given");
+  }
+  p.positions = positions.data_ptr<int64_t>();
+  p.talk = nullptr;
+  if (talk.has_value()) {
+    CHECK_GPU(*talk); CHECK_CONTIG(*talk); CHECK_F32(*talk);
+    TORCH_CHECK(talk->numel() == H * H, "talking_attention: talk must be [H, H]");
+    p.talk = talk->data_ptr<float>();
+  }
+  p.gate = nullptr; p.gate_stride = 0;
+  if (gate.has_value()) {
+    CHECK_GPU(*gate); CHECK_LAST_CONTIG(*gate);
+    TORCH_CHECK(gate->dim() == 2 && gate->size(0) == T && gate->size(1) == H * Dv &&
+                    gate->scalar_type() == q.scalar_type(), "talking_attention: gate [T, H Dv]");
+    p.gate = gate->data_ptr(); p.gate_stride = gate->stride(0);
+  }
+  p.scale = (float)scale;
+  p.T = T; p.H = H; p.G = G; p.D = D; p.Dv = Dv; p.BS = BS;
+  p.ws_ml = nullptr; p.ws_o = nullptr; p.num_parts = 1;
+  if (num_parts > 1) {
+    TORCH_CHECK(ws_ml.has_value() && ws_o.has_value(), "talking_attention: a workspace for parts");
+    CHECK_GPU(*ws_ml); CHECK_GPU(*ws_o); CHECK_F32(*ws_ml); CHECK_F32(*ws_o);
+    TORCH_CHECK(ws_ml->numel() >= T * num_parts * H * 2 &&
+                    ws_o->numel() >= T * num_parts * H * G * Dv, "talking_attention: workspace size");
+    p.ws_ml = ws_ml->data_ptr<float>(); p.ws_o = ws_o->data_ptr<float>();
+    p.num_parts = num_parts;
+    TORCH_CHECK((num_parts + 1) * H * 4 <= 65536, "talking_attention: too many partitions");
+  }
+  TORCH_CHECK(akap_stream::talking_attention_lds(H, D) <= 65536,
+              "talking_attention: heads x head size too large for the query row in LDS");
+  const c10::DeviceGuard g(q.device());
+  akap_stream::launch_talking_attention(p, f32, cur_stream());
+}
+
+void route_topk(Tensor ids, Tensor w, Tensor h, Tensor router, std::optional<Tensor> bias) {
+  CHECK_GPU(ids); CHECK_GPU(w); CHECK_GPU(h); CHECK_GPU(router);
+  CHECK_CONTIG(ids); CHECK_CONTIG(w); CHECK_F32(w); CHECK_LAST_CONTIG(h); CHECK_CONTIG(router);
+  CHECK_F32(router);
+  TORCH_CHECK(h.dim() == 2 && router.dim() == 2 && router.size(1) == h.size(1), "route_topk: shapes");
+  const int64_t T = h.size(0), n = router.size(0);
+  TORCH_CHECK(ids.scalar_type() == at::kInt && ids.dim() == 2 && ids.size(0) == T &&
+                  w.sizes() == ids.sizes() && ids.size(1) >= 1 && ids.size(1) <= n && n <= 8192,
+              "route_topk: ids / w");
+  const float* bp = nullptr;
+  if (bias.has_value()) {
+    CHECK_GPU(*bias); CHECK_CONTIG(*bias); CHECK_F32(*bias);
+    TORCH_CHECK(bias->numel() == n, "route_topk: bias");
+    bp = bias->data_ptr<float>();
+  }
+  const c10::DeviceGuard g(h.device());
+  akap_stream::launch_route_topk(ids.data_ptr<int32_t>(), w.data_ptr<float>(), h.data_ptr(),
+                                 (int)h.stride(0), router.data_ptr<float>(), bp, (int)T,
+                                 (int)h.size(1), (int)n, (int)ids.size(1), is_f32(h, "h"),
+                                 cur_stream());
+}
+
+void swiglu_routed(Tensor out, Tensor gu, std::optional<Tensor> ids, std::optional<Tensor> w,
+                   int64_t experts) {
+  CHECK_GPU(out); CHECK_GPU(gu); CHECK_LAST_CONTIG(out); CHECK_LAST_CONTIG(gu);
+  TORCH_CHECK(out.scalar_type() == gu.scalar_type() && out.dim() == 2 && gu.dim() == 2 &&
+                  out.size(0) == gu.size(0) && experts >= 1 && gu.size(1) == 2 * out.size(1) &&
+                  out.size(1) % experts == 0 && experts <= 8192, "swiglu_routed: shapes");
+  const int64_t T = gu.size(0);
+  const int32_t* ip = nullptr;
+  const float* wp = nullptr;
+  int top = 0;
+  if (ids.has_value()) {
+    TORCH_CHECK(w.has_value(), "swiglu_routed: ids need weights");
+    CHECK_GPU(*ids); CHECK_GPU(*w); CHECK_CONTIG(*ids); CHECK_CONTIG(*w); CHECK_F32(*w);
+    TORCH_CHECK(ids->scalar_type() == at::kInt && ids->dim() == 2 && ids->size(0) == T &&
+                    w->sizes() == ids->sizes() && ids->size(1) <= 256, "swiglu_routed: ids / w");
+    ip = ids->data_ptr<int32_t>(); wp = w->data_ptr<float>(); top = ids->size(1);
+  }
+  const c10::DeviceGuard g(gu.device());
+  akap_stream::launch_swiglu_routed(out.data_ptr(), (int)out.stride(0), gu.data_ptr(),
+                                    (int)gu.stride(0), ip, wp, (int)T, top, (int)experts,
+                                    (int)(out.size(1) / experts), is_f32(gu, "gu"), cur_stream());
+}
+
 }  // namespace
 
 TORCH_LIBRARY(akap_stream, m) {
@@ -730,6 +972,19 @@ TORCH_LIBRARY(akap_stream, m) {
   m.def("relu2_routed(Tensor(a!) out, Tensor up, Tensor ids, Tensor w, int experts) -> ()");
   m.def("moe_combine(Tensor(a!) out, Tensor y, Tensor? inv, Tensor ids, Tensor w, Tensor h, "
         "int experts) -> ()");
+  m.def("post_norm_add_norm(Tensor(a!) out, Tensor(b!) x, Tensor ya, Tensor? yb, Tensor? wa, "
+        "Tensor? wb, Tensor post_w, Tensor next_w, float eps, bool fresh) -> ()");
+  m.def("head_norm_cache(Tensor proj, Tensor(a!) q_out, Tensor(b!) k_cache, Tensor(c!) v_cache, "
+        "Tensor slots, int H, int G, int D, int Dv, int q_off, int k_off, int v_off, float eps, "
+        "bool norm_qk, bool norm_v) -> ()");
+  m.def("retention(Tensor(a!) out, Tensor proj, int q_off, int k_off, int v_off, int g_off, "
+        "Tensor(b!) state, Tensor seq_slot, Tensor positions, Tensor? q_start, Tensor? cos_sin, "
+        "Tensor log2_decay, int H, int D, int V, float eps) -> ()");
+  m.def("talking_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, "
+        "Tensor block_tables, Tensor seq_lens, Tensor? q_start, Tensor positions, Tensor? talk, "
+        "Tensor? gate, float scale, Tensor(b!)? ws_ml, Tensor(c!)? ws_o, int num_parts) -> ()");
+  m.def("route_topk(Tensor(a!) ids, Tensor(b!) w, Tensor h, Tensor router, Tensor? bias) -> ()");
+  m.def("swiglu_routed(Tensor(a!) out, Tensor gu, Tensor? ids, Tensor? w, int experts) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(akap_stream, CUDA, m) {
@@ -746,6 +1001,12 @@ TORCH_LIBRARY_IMPL(akap_stream, CUDA, m) {
   m.impl("moe_route", &moe_route);
   m.impl("relu2_routed", &relu2_routed);
   m.impl("moe_combine", &moe_combine);
+  m.impl("post_norm_add_norm", &post_norm_add_norm);
+  m.impl("head_norm_cache", &head_norm_cache);
+  m.impl("retention", &retention);
+  m.impl("talking_attention", &talking_attention);
+  m.impl("route_topk", &route_topk);
+  m.impl("swiglu_routed", &swiglu_routed);
   m.impl("embed_scaled", &embed_scaled);
   m.impl("add_norm", &add_norm);
   m.impl("relu2", &relu2);

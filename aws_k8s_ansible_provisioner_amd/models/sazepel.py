@@ -306,11 +306,12 @@ class SazepelLM:
         return ks, vs
 
     def allocate_state(self, num_slots: int) -> None:
-        """The retention state per layer run and sequence slot: [slots, H, D, V] fp32."""
+        """The retention state per layer run and sequence slot, transposed: [slots, H, V, D]
+        fp32."""
         self.state = []
         for i in self.runs:
             _, r = self._parts(self.cfg.layer_specs[i])
-            self.state.append(torch.zeros(max(1, num_slots), r.heads, r.dim, r.vdim,
+            self.state.append(torch.zeros(max(1, num_slots), r.heads, r.vdim, r.dim,
                                           dtype=torch.float32, device=self.device))
 
     def state_bytes_per_slot(self) -> int:

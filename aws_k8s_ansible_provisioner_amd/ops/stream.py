@@ -786,8 +786,8 @@ def retention(out: torch.Tensor, proj: torch.Tensor, q_off: int, k_off: int, v_o
     layout (i pairs with i + dims/2) by the angle row of positions[t]; k is scaled by D^-1/2;
     S <- decay_h S + k v^T and o = S^T q with decay_h = 2^log2_decay[h]; o is divided by its
     root mean square over V (eps inside the root) and multiplied by silu(g):
-    out[t, h V : (h + 1) V].  The state S [D, V] (fp32) of a sequence lives in
-    state[slot, h]: the rows of sequence b are [q_start[b], q_start[b + 1]) (q_start None: row
+    out[t, h V : (h + 1) V].  The state of a sequence lives TRANSPOSED in state[slot, h]
+    (fp32 [V, D] = S^T: the D entries a GPU thread keeps in registers are contiguous): the rows of sequence b are [q_start[b], q_start[b + 1]) (q_start None: row
     t is a sequence of its own), its slot is seq_slot of its first row (-1: padding, nothing
     is read or written); it starts from zeros when its first row has position 0, else from
     what an earlier step left in the slot, and the state after its last row is written back.
@@ -816,12 +816,12 @@ def retention(out: torch.Tensor, proj: torch.Tensor, q_off: int, k_off: int, v_o
         if r1 <= r0 or int(seq_slot[r0]) < 0:
             continue
         slot = int(seq_slot[r0])
-        S = state[slot].float().clone() if int(positions[r0]) > 0 else \
+        S = state[slot].float().transpose(1, 2).clone() if int(positions[r0]) > 0 else \
             torch.zeros(H, D, V, dtype=torch.float32)
         for t in range(r0, r1):
             S = decay * S + k[t][:, :, None] * v[t][:, None, :]
             o[t] = torch.einsum("hdv,hd->hv", S, q[t])
-        state[slot] = S
+        state[slot] = S.transpose(1, 2)
         on = _rms(o[r0:r1], eps) * torch.nn.functional.silu(g[r0:r1])
         out[r0:r1] = on.reshape(r1 - r0, H * V).to(out.dtype)
 

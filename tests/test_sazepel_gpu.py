@@ -1,0 +1,203 @@
+"""Sazepel on the HIP kernels: every new kernel against the PyTorch version of the same op (fp32
+and bf16 storage, odd sizes), then the engine -- mixed steps, hipGraph decode, a small page and
+slot pool -- against the float64 oracle (tests/sazepel_oracle.py), and greedy generation
+through LLMEngine.generate."""
+import pytest
+import torch
+
+from aws_k8s_ansible_provisioner_amd.ops import stream as sops
+
+pytestmark = pytest.mark.gpu
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def close(a, b, dtype, scale=1.0):
+    tol = 3e-5 if dtype == "float32" else 2e-2
+    torch.testing.assert_close(a.float().cpu(), b.float().cpu(), rtol=tol, atol=tol * scale)
+
+
+# ------------------------------------------------------------------ kernels against their ops
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("d", [24, 200, 2048, 4100, 8192])
+def test_post_norm_add_norm_kernel(dtype, d):
+    g, dt = gen(d), DT[dtype]
+    T = 5
+    x = torch.randn(T, d, generator=g)
+    ya = torch.randn(T, d + 8, generator=g).to(dt)[:, :d]
+    yb = (3 * torch.randn(T, d, generator=g)).to(dt)
+    y32 = torch.randn(T, d, generator=g)
+    wa, wb = 1 + 0.3 * torch.randn(d, generator=g), 1 + 0.3 * torch.randn(d, generator=g)
+    one, vec = torch.tensor([0.7]), 1 + 0.3 * torch.randn(d, generator=g)
+    cases = [(ya, None, None, None, one, one, False), (ya, yb, wa, wb, one, vec, False),
+             (y32, None, None, None, vec, one, False), (ya, None, None, None, one, one, True),
+             (ya, yb, one, one, vec, vec, True)]
+    for a, b, u, v, pw, nw, fresh in cases:
+        res = []
+        for dev in ("cpu", "cuda"):
+            mv = lambda t: None if t is None else t.to(dev)  # noqa: E731
+            xx = x.clone().to(dev) if not fresh else torch.full((T, d), 9.0, device=dev)
+            o = torch.zeros(T, d, dtype=dt, device=dev)
+            sops.stream_post_norm_add_norm(xx, mv(a), mv(b), mv(u), mv(v), mv(pw), mv(nw), 1e-6, o,
+                                           fresh=fresh)
+            res.append((xx, o))
+        close(res[1][0], res[0][0], "float32")
+        close(res[1][1], res[0][1], dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,G,D,Dv", [(6, 3, 96, 96), (4, 1, 20, 36), (8, 8, 128, 64), (3, 3, 7, 5)])
+def test_head_norm_cache_kernel(dtype, H, G, D, Dv):
+    g, dt = gen(H * D), DT[dtype]
+    T, NB, BS = 9, 4, 16
+    N = H * D + G * (D + Dv) + 11
+    proj = torch.randn(T, N, generator=g).to(dt)
+    slots = torch.tensor([5, 17, 63, 0, -1, 33, 16, 15, 48])
+    res = []
+    for dev in ("cpu", "cuda"):
+        for nq, nv in ((True, True), (False, True), (True, False)):
+            q = torch.zeros(T, H, D, dtype=dt, device=dev)
+            kc = torch.zeros(NB, G, BS, D, dtype=dt, device=dev)
+            vc = torch.zeros(NB, G, BS, Dv, dtype=dt, device=dev)
+            sops.head_norm_cache(proj.to(dev), q, kc, vc, slots.to(dev), H, G, D, Dv, 3, 3 + H * D,
+                                 3 + H * D + G * D, 1e-6, nq, nv)
+            res.append((q, kc, vc))
+    n = len(res) // 2
+    for i in range(n):
+        for a, b in zip(res[i], res[n + i]):
+            close(b, a, dtype)
+
+
+def _retention_case(dtype, H, D, V, rot, dev, steps, g, slots=3):
+    """Run `steps` (each a list of (slot, first position, rows)) through the op; returns the
+    outputs of all steps and the final state."""
+    dt = DT[dtype]
+    N = H * (2 * D + 2 * V) + 5
+    state = torch.zeros(slots, H, V, D, device=dev)
+    decay = torch.log2(torch.tensor([0.9 + 0.099 * h / max(1, H - 1) for h in range(H)]))
+    cs = sops.rotary_table(512, rot, 10000.0) if rot else None
+    outs = []
+    for step in steps:
+        T = sum(n for _, _, n in step)
+        proj = torch.randn(T, N, generator=g).to(dt)
+        slot = torch.cat([torch.full((n,), s, dtype=torch.int32) for s, _, n in step])
+        pos = torch.cat([torch.arange(p, p + n) for _, p, n in step])
+        qs = torch.tensor([0] + [n for _, _, n in step], dtype=torch.int32).cumsum(0).int()
+        single = all(n == 1 for _, _, n in step)
+        out = torch.zeros(T, H * V + 3, dtype=dt, device=dev)
+        sops.retention(out[:, :H * V], proj.to(dev), 2, 2 + H * D, 2 + 2 * H * D,
+                       2 + 2 * H * D + H * V, state, slot.to(dev), pos.to(dev),
+                       None if single else qs.to(dev), cs.to(dev) if rot else None,
+                       decay.to(dev), H, D, V, 1e-6)
+        outs.append(out)
+    return outs, state
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,D,V,rot", [(4, 64, 64, 64), (4, 64, 32, 32), (2, 128, 128, 64),
+                                       (3, 24, 40, 8), (2, 80, 96, 0), (1, 256, 256, 128),
+                                       (2, 16, 8, 16)])
+def test_retention_kernel(dtype, H, D, V, rot):
+    # portions of several sequences, a sequence continued from its slot, single rows, a slot
+    # started again at position 0 over what an earlier sequence left, a padding row
+    steps = [[(0, 0, 37), (2, 0, 3)], [(0, 37, 1), (2, 3, 1)], [(2, 4, 18), (0, 38, 2), (-1, 0, 1)],
+             [(1, 0, 1), (0, 40, 1)], [(2, 0, 5)]]
+    res = [_retention_case(dtype, H, D, V, rot, dev, steps, gen(7)) for dev in ("cpu", "cuda")]
+    for a, b in zip(res[0][0], res[1][0]):
+        close(b, a, dtype, scale=3.0)
+    close(res[1][1], res[0][1], "float32")
+
+
+def _attention_case(dtype, H, G, D, Dv, dev, g, parts, talk=True, gate=True, BS=16):
+    dt = DT[dtype]
+    lens = [70, 1, 33, 130]                     # cached keys per sequence
+    rows = [5, 1, 33, 1]                        # rows of this step (the last positions)
+    NB = sum(-(-n // BS) for n in lens) + 2
+    kc = torch.randn(NB, G, BS, D, generator=g).to(dt)
+    vc = torch.randn(NB, G, BS, Dv, generator=g).to(dt)
+    perm = torch.randperm(NB, generator=g).int()
+    mb = max(-(-n // BS) for n in lens)
+    bt = torch.zeros(len(lens), mb, dtype=torch.int32)
+    o = 0
+    for b, n in enumerate(lens):
+        nb = -(-n // BS)
+        bt[b, :nb] = perm[o:o + nb]
+        o += nb
+    T = sum(rows)
+    q = torch.randn(T, H, D, generator=g).to(dt)
+    pos = torch.cat([torch.arange(n - r, n) for n, r in zip(lens, rows)])
+    qs = torch.tensor([0] + rows, dtype=torch.int32).cumsum(0).int()
+    tk = (torch.eye(H) + 0.3 * torch.randn(H, H, generator=g)) if talk else None
+    gt = torch.randn(T, H * Dv + 4, generator=g).to(dt)[:, 2:2 + H * Dv] if gate else None
+    out = torch.zeros(T, H * Dv + 8, dtype=dt, device=dev)
+    mv = lambda t: None if t is None else t.to(dev)  # noqa: E731
+    ws = sops.talking_attention_workspace(T, H, G, Dv, parts, dev) if parts > 1 else None
+    sops.talking_attention(out[:, :H * Dv], mv(q), mv(kc), mv(vc), mv(bt),
+                           torch.tensor(lens, dtype=torch.int32, device=dev), mv(qs), mv(pos),
+                           mv(tk), mv(gt), 0.3, ws, parts)
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,G,D,Dv", [(6, 3, 96, 96), (4, 1, 20, 36), (8, 8, 32, 64),
+                                      (16, 4, 128, 128), (5, 5, 8, 200)])
+def test_talking_attention_kernel(dtype, H, G, D, Dv):
+    want = _attention_case(dtype, H, G, D, Dv, "cpu", gen(3), 1)
+    for parts in (1, 2, 5):
+        close(_attention_case(dtype, H, G, D, Dv, "cuda", gen(3), parts), want, dtype)
+    want = _attention_case(dtype, H, G, D, Dv, "cpu", gen(4), 1, talk=False, gate=False)
+    close(_attention_case(dtype, H, G, D, Dv, "cuda", gen(4), 3, talk=False, gate=False), want,
+          dtype)
+
+
+def test_talking_attention_decode_rows_without_sequence_starts():
+    # one row per sequence (a decode step), a padding sequence among them
+    g = gen(11)
+    H, G, D, Dv, BS = 4, 2, 32, 16, 32
+    lens = torch.tensor([40, 0, 200, 1], dtype=torch.int32)
+    NB = 12
+    kc, vc = torch.randn(NB, G, BS, D, generator=g), torch.randn(NB, G, BS, Dv, generator=g)
+    bt = torch.tensor([[0, 1, 0, 0, 0, 0, 0], [0] * 7, [2, 3, 4, 5, 6, 7, 8], [9, 0, 0, 0, 0, 0, 0]],
+                      dtype=torch.int32)
+    q = torch.randn(4, H, D, generator=g)
+    pos = (lens - 1).clamp(min=0).long()
+    tk, gt = torch.randn(H, H, generator=g), torch.randn(4, H * Dv, generator=g)
+    outs = []
+    for dev, parts in (("cpu", 1), ("cuda", 1), ("cuda", 4)):
+        out = torch.full((4, H * Dv), 7.0, device=dev)
+        ws = sops.talking_attention_workspace(4, H, G, Dv, parts, dev) if parts > 1 else None
+        sops.talking_attention(out, q.to(dev), kc.to(dev), vc.to(dev), bt.to(dev), lens.to(dev),
+                               None, pos.to(dev), tk.to(dev), gt.to(dev), 0.2, ws, parts)
+        outs.append(out)
+    assert (outs[0][1] == 7.0).all() and (outs[1][1] == 7.0).all() and (outs[2][1] == 7.0).all()
+    close(outs[1], outs[0], "float32")
+    close(outs[2], outs[0], "float32")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("E,top,F_,d", [(16, 3, 96, 192), (5, 5, 7, 40), (8, 1, 64, 256), (3, 2, 8, 24)])
+def test_routing_and_gated_activation_kernels(dtype, E, top, F_, d):
+    g, dt = gen(E * d), DT[dtype]
+    T = 13
+    h = torch.randn(T, d, generator=g).to(dt)
+    router, bias = torch.randn(E, d, generator=g), torch.randn(E, generator=g)
+    ids_c, w_c = sops.route_topk(h, router, bias, top)
+    ids_g, w_g = sops.route_topk(h.cuda(), router.cuda(), bias.cuda(), top)
+    assert (ids_g.cpu() == ids_c).all()
+    close(w_g, w_c, "float32")
+    ids_n, w_n = sops.route_topk(h.cuda(), router.cuda(), None, top)
+    want = sops.route_topk(h, router, None, top)
+    assert (ids_n.cpu() == want[0]).all()
+    gu = torch.randn(T, E * 2 * F_ + 8, generator=g).to(dt)[:, :E * 2 * F_]
+    a_c = torch.zeros(T, E * F_, dtype=dt)
+    a_g = torch.zeros(T, E * F_, dtype=dt, device="cuda")
+    sops.swiglu_routed(gu, ids_c, w_c, E, a_c)
+    sops.swiglu_routed(gu.cuda(), ids_g, w_g, E, a_g)
+    close(a_g, a_c, dtype)
+    s_c, s_g = torch.zeros(T, E * F_, dtype=dt), torch.zeros(T, E * F_, dtype=dt, device="cuda")
+    sops.swiglu(gu[:, :2 * E * F_], s_c)
+    sops.swiglu(gu.cuda()[:, :2 * E * F_], s_g)
+    close(s_g, s_c, dtype)
