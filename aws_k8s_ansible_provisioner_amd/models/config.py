@@ -735,6 +735,40 @@ TINY_PUPUTAR = register(_puputar_stack(
     norm_groups=4))
 
 
+def _sazepel_stack(name: str, width: int, n: int, att: tuple, ret: tuple, experts: int,
+                   expert_ff: int, top: int, vocab: int = 32000, rot_dims: Optional[int] = None,
+                   logit_scale: float = 1.0) -> LayeredConfig:
+    """n layers; every third one (from the second) is a retention alone, the others put an
+    attention beside it; the last layer has no feed-forward."""
+    layers = []
+    for i in range(n):
+        ly = dict(ret=ret, base=500000.0)
+        if rot_dims is not None:
+            ly["rot_dims"] = rot_dims
+        if i % 3 != 1:
+            ly["att"] = att
+        if i + 1 < n:
+            ly.update(experts=experts, expert_ff=expert_ff, top=top)
+        layers.append(ly)
+    cfg = sazepel_config(name, sazepel_dict(width, layers, vocab=vocab, logit_scale=logit_scale))
+    cfg.hf_id = "test/" + name
+    return cfg
+
+
+# Sazepel at layer sizes of real models (random weights; bench.py --compare-design sazepel):
+# 16 / 4 attention heads of 128 beside 8 retention heads with 128 x 128 states, 8 experts of
+# which 2 per token
+SAZEPEL_W2048 = register(_sazepel_stack(
+    "sazepel-w2048", width=2048, n=16, att=(16, 4, 128, 128), ret=(8, 128, 128), experts=8,
+    expert_ff=1408, top=2, rot_dims=64))
+SAZEPEL_W4096 = register(_sazepel_stack(
+    "sazepel-w4096", width=4096, n=8, att=(32, 8, 128, 128), ret=(16, 128, 128), experts=8,
+    expert_ff=3584, top=2, rot_dims=64))
+TINY_SAZEPEL = register(_sazepel_stack(
+    "tiny-sazepel", width=128, n=4, att=(4, 2, 32, 16), ret=(2, 16, 32), experts=6, expert_ff=64,
+    top=2, vocab=512, rot_dims=8, logit_scale=1.5))
+
+
 def get_config(name: str) -> ModelConfig:
     """Resolve a registry name, HF id, or a directory holding a HF config.json."""
     if os.path.isdir(name) and os.path.exists(os.path.join(name, "config.json")):

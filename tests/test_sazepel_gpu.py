@@ -5,10 +5,14 @@ through LLMEngine.generate."""
 import pytest
 import torch
 
+import sazepel_oracle as oracle
+from bidetar_harness import engine, rel_err, replay, tokens, write_model
+from test_sazepel import OTHER, base_config
 from aws_k8s_ansible_provisioner_amd.ops import stream as sops
 
 pytestmark = pytest.mark.gpu
 DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+TOL = {"float32": 3e-4, "bfloat16": 0.3}
 
 
 def gen(seed):
@@ -201,3 +205,135 @@ def test_routing_and_gated_activation_kernels(dtype, E, top, F_, d):
     sops.swiglu(gu[:, :2 * E * F_], s_c)
     sops.swiglu(gu.cuda()[:, :2 * E * F_], s_g)
     close(s_g, s_c, dtype)
+
+
+# ------------------------------------------------------------------ the engine on the GPU
+@pytest.fixture(scope="module")
+def model(tmp_path_factory):
+    cfg = base_config()
+    W = oracle.random_weights(cfg, seed=2)
+    reqs = {"a": tokens(75, cfg["vocab"], 1), "b": tokens(41, cfg["vocab"], 2),
+            "c": tokens(23, cfg["vocab"], 3), "d": tokens(1, cfg["vocab"], 4),
+            "e": tokens(64, cfg["vocab"], 5)}
+    want = {n: oracle.forward(cfg, W, t) for n, t in reqs.items()}
+    return cfg, W, write_model(tmp_path_factory.mktemp("sazepel_gpu"), cfg, W), reqs, want
+
+
+def check(got, want, dtype):
+    for n in got:
+        e = rel_err(got[n], want[n])
+        if dtype == "bfloat16":
+            # widths of a few dozen make bf16 rounding large against the logits and a close
+            # routing choice can flip: the bulk of the positions must be close
+            assert e.median().item() < 0.15, f"{n}: median {e.median():.2e}, worst {e.max():.2e}"
+        else:
+            assert e.max().item() < TOL[dtype], f"{n}: position {int(e.argmax())} off by {e.max():.2e}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("eager", [False, True])
+def test_schedules(model, dtype, eager):
+    _, _, path, reqs, want = model
+    eng = engine(path, dtype=dtype, device="cuda", eager=eager)
+    assert eager or eng.runner.graphs, "decode hipGraphs were not captured"
+    one = {"a": reqs["a"]}
+    check(replay(eng, reqs, [[(n, len(t))] for n, t in reqs.items()]), want, dtype)
+    check(replay(eng, one, [[("a", 40)]] + [[("a", 1)]] * 35), want, dtype)
+    check(replay(eng, one, [[("a", s)] for s in [3, 2, 7, 2, 19, 2, 5, 33, 2]]), want, dtype)
+    sched = [[("a", 30), ("b", 2), ("c", 1)],
+             [("a", 1), ("b", 20), ("c", 22), ("d", 1)],
+             [("a", 1), ("b", 1), ("e", 33)],
+             [("a", 1), ("b", 1)],
+             [("b", 17), ("e", 1)],
+             [("a", 42), ("e", 30)]]
+    check(replay(eng, reqs, sched), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_small_pool_is_used_again(model, dtype):
+    _, _, path, reqs, want = model
+    eng = engine(path, dtype=dtype, max_tokens=160, max_seqs=2, device="cuda")
+    many = {f"{n}{i}": reqs[n] for i in range(2) for n in ("b", "c", "e")}
+    many["a"] = reqs["a"]
+    sched = [[("b0", 41), ("c0", 23)], [("e0", 64), ("c1", 22)], [("c1", 1)],
+             [("a", 75), ("b1", 41)], [("e1", 10)], [("e1", 54)]]
+    for _ in range(2):  # graphs replayed again over pages and slots that changed owners
+        check(replay(eng, many, sched), {k: want[k[0]] for k in many}, dtype)
+    assert eng.sched.num_free_blocks() == 5 and eng.sched.num_free_tail_slots == 2
+
+
+def test_long_decode_through_graphs(tmp_path):
+    """Decoding far past the first key partition of the split attention, the retention state
+    carried by the captured graphs."""
+    cfg = oracle.make_config(width=64, vocab=37, logit_scale=0.8, layers=[
+        oracle.make_layer(oracle.ret_spec(2, 16, 16, rot_dims=8, decay=[0.999, 0.97]),
+                          att=(4, 2, 16, 8, 0.25), moe=(6, 2, 16)),
+        oracle.make_layer(oracle.ret_spec(4, 8, 12, decay=[1.0, 0.995, 0.9, 0.6]))])
+    W = oracle.random_weights(cfg, seed=5)
+    toks = tokens(700, 37, 6)
+    want = {"a": oracle.forward(cfg, W, toks)}
+    eng = engine(write_model(tmp_path, cfg, W), dtype="float32", max_tokens=704, device="cuda")
+    assert eng.runner.graphs
+    check(replay(eng, {"a": toks}, [[("a", 500)]] + [[("a", 1)]] * 200), want, "float32")
+
+
+def test_large_prompt_takes_the_sorted_expert_path(tmp_path):
+    """A prompt portion over the small-batch threshold of the routed feed-forward."""
+    from aws_k8s_ansible_provisioner_amd.models import sazepel
+
+    cfg = oracle.make_config(width=32, vocab=37, layers=[
+        oracle.make_layer(oracle.ret_spec(2, 8, 8, rot_dims=4), att=(2, 1, 8, 8, 0.4),
+                          moe=(5, 2, 16))])
+    W = oracle.random_weights(cfg, seed=6)
+    toks = tokens(sazepel.MOE_DENSE_ROWS + 70, 37, 7)
+    want = {"a": oracle.forward(cfg, W, toks)}
+    eng = engine(write_model(tmp_path, cfg, W), dtype="float32", max_tokens=512, device="cuda")
+    n = sazepel.MOE_DENSE_ROWS + 40
+    check(replay(eng, {"a": toks}, [[("a", n)], [("a", 30)]]), want, "float32")
+
+
+def test_greedy_generation(model):
+    from aws_k8s_ansible_provisioner_amd.engine.config import EngineConfig, SamplingParams
+    from aws_k8s_ansible_provisioner_amd.engine.llm_engine import LLMEngine
+
+    cfg, W, path, _, _ = model
+    eng = LLMEngine(EngineConfig(model=path, load_format="safetensors", weights_path=path,
+                                 dtype="float32", max_model_len=128, max_num_seqs=4,
+                                 max_num_batched_tokens=24, num_gpu_blocks=16, device="cuda",
+                                 gc_freeze=False), log=lambda *a: None)
+    assert eng.runner.graphs
+    prompts = [tokens(n, cfg["vocab"], 20 + n) for n in (30, 3, 17, 9)]
+    outs = eng.generate(None, SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True),
+                        prompt_ids=prompts)
+    assert [len(o.output_ids) for o in outs] == [12] * 4
+    for p, o in zip(prompts, outs):
+        logits = oracle.forward(cfg, W, p + o.output_ids)
+        for i, tok in enumerate(o.output_ids):
+            row = logits[len(p) - 1 + i]
+            assert row[tok] >= row.max() - 1e-3 * row.std(), (i, tok, int(row.argmax()))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(OTHER))
+def test_other_configurations(tmp_path, name, dtype):
+    cfg = oracle.make_config(**dict({"vocab": 31}, **OTHER[name]))
+    W = oracle.random_weights(cfg, seed=len(name))
+    reqs = {"p": tokens(45, cfg["vocab"], 11), "q": tokens(38, cfg["vocab"], 12)}
+    want = {n: oracle.forward(cfg, W, t) for n, t in reqs.items()}
+    eng = engine(write_model(tmp_path, cfg, W), dtype=dtype, device="cuda")
+    sched = [[("p", 17), ("q", 2)], [("p", 1), ("q", 30)], [("p", 27), ("q", 1)],
+             [("q", 1)], [("q", 4)]]
+    check(replay(eng, reqs, sched), want, dtype)
+
+
+def test_registry_model_generates_with_sampling():
+    from aws_k8s_ansible_provisioner_amd.engine.config import EngineConfig, SamplingParams
+    from aws_k8s_ansible_provisioner_amd.engine.llm_engine import LLMEngine
+
+    eng = LLMEngine(EngineConfig(model="tiny-sazepel", dtype="bfloat16", max_model_len=256,
+                                 max_num_seqs=4, max_num_batched_tokens=64, num_gpu_blocks=32,
+                                 device="cuda", gc_freeze=False), log=lambda *a: None)
+    outs = eng.generate(None, SamplingParams(max_tokens=20, temperature=0.8, top_p=0.9, seed=3,
+                                             ignore_eos=True),
+                        prompt_ids=[[5, 6, 7], [9] * 70, [1, 2], [3] * 33, [4] * 5])
+    assert [len(o.output_ids) for o in outs] == [20] * 5
