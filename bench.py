@@ -89,7 +89,7 @@ def parse():
                          "kernel table")
     ap.add_argument("--profile-steps", type=int, default=0,
                     help="extra untimed waves run after timing (for rocprofv3 captures)")
-    ap.add_argument("--compare-design", default=None, choices=["bidetar", "puputar"],
+    ap.add_argument("--compare-design", default=None, choices=["bidetar", "puputar", "sazepel"],
                     help="instead of the serving wave: prefill and decode throughput of this "
                          "design at real layer sizes (random weights) beside the closest "
                          "existing model of equal size; prints one JSON line with the table")
@@ -106,6 +106,11 @@ COMPARE_SETS = {
     # latent attention + token shift beside the framework's other fp32-stream design at the
     # same width, depth and head count; the routed variant has no equal-size counterpart
     "puputar": [("puputar-w2048", "bidetar-w2048"), ("puputar-w4096", "bidetar-w4096"),
+                ("puputar-w2048-moe", None)],
+    # retention + head-mixed attention + routed SwiGLU experts beside the framework's other
+    # fp32-stream designs at the same width and depth: the dense one with softmax attention
+    # and the one with routed experts
+    "sazepel": [("sazepel-w2048", "bidetar-w2048"), ("sazepel-w4096", "bidetar-w4096"),
                 ("puputar-w2048-moe", None)],
 }
 
