@@ -24,6 +24,18 @@ __device__ __forceinline__ void stf(T* p, float v) { *p = (T)v; }
 
 __device__ __forceinline__ float sigmoidf(float z) { return 1.0f / (1.0f + __expf(-z)); }
 
+// 8 consecutive elements (32- resp. 16-byte aligned) as floats
+__device__ __forceinline__ void ld8(const float* p, float (&v)[8]) {
+  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+  v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void ld8(const bf16* p, float (&v)[8]) {
+  const akap::bf16x8 a = *(const akap::bf16x8*)p;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = (float)a[i];
+}
+
 // ------------------------------------------------------------------ post-norm + residual + norm
 // one workgroup per row; a thread keeps to its own columns in every phase, so the two LDS rows
 // need no barrier beyond those of the block sums
@@ -93,7 +105,7 @@ __global__ __launch_bounds__(256) void head_norm_cache_kernel(HeadNormParams p) 
   for (int u = wave; u < p.H + 2 * p.G; u += 4) {
     const T* src;
     T* dst;
-    int n;
+    int n, vstep = 1;
     bool norm;
     if (u < p.H) {
       src = row + p.q_off + u * p.D;
@@ -111,9 +123,13 @@ __global__ __launch_bounds__(256) void head_norm_cache_kernel(HeadNormParams p) 
       if (!cached) continue;
       const int g = u - p.H - p.G;
       src = row + p.v_off + g * p.Dv;
-      dst = (T*)p.v_cache + ((size_t)(blk * p.G + g) * p.BS + off) * p.Dv;
+      // values go in groups of 8 tokens, dimension-major inside a group: entry c of token
+      // `off` sits at [off / 8][c][off % 8]
+      dst = (T*)p.v_cache + (((size_t)(blk * p.G + g) * (p.BS >> 3) + (off >> 3)) * p.Dv) * 8 +
+            (off & 7);
       n = p.Dv;
       norm = p.norm_v;
+      vstep = 8;
     }
     float inv = 1.0f;
     if (norm) {
@@ -125,7 +141,7 @@ __global__ __launch_bounds__(256) void head_norm_cache_kernel(HeadNormParams p) 
       ss = wave_sum(ss);
       inv = 1.0f / sqrtf(ss / (float)n + p.eps);
     }
-    for (int c = lane; c < n; c += 64) stf(dst + c, ldf(src + c) * inv);
+    for (int c = lane; c < n; c += 64) stf(dst + c * vstep, ldf(src + c) * inv);
   }
 }
 
@@ -342,7 +358,19 @@ __global__ __launch_bounds__(1024) void talking_attention_kernel(TalkParams p) {
         float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
         const float* q0 = qs + (kc * rep + i0) * p.D;
         const int n = min(4, rep - i0);
-        if (live) {
+        if (live && (p.D & 7) == 0) {
+          for (int d = 0; d < p.D; d += 8) {
+            float k8[8];
+            ld8(kr + d, k8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              s0 = fmaf(q0[d + e], k8[e], s0);
+              if (n > 1) s1 = fmaf(q0[p.D + d + e], k8[e], s1);
+              if (n > 2) s2 = fmaf(q0[2 * p.D + d + e], k8[e], s2);
+              if (n > 3) s3 = fmaf(q0[3 * p.D + d + e], k8[e], s3);
+            }
+          }
+        } else if (live) {
           for (int d = 0; d < p.D; ++d) {
             const float kv = ldf(kr + d);
             s0 = fmaf(q0[d], kv, s0);
@@ -375,29 +403,32 @@ __global__ __launch_bounds__(1024) void talking_attention_kernel(TalkParams p) {
       for (int g = 0; g < HMAX; ++g)
         if (g < p.H) acc[g] *= alpha[g];
       const int nk = min(TA_PIECE, hi - j0);
-      const T* vb = (const T*)p.v_cache + (size_t)c * p.BS * p.Dv + dv;
-      int jj = 0;
-      for (; jj + 4 <= nk; jj += 4) {
-        const float v0 = ldf(vb + (size_t)rowbase[jj] * p.Dv);
-        const float v1 = ldf(vb + (size_t)rowbase[jj + 1] * p.Dv);
-        const float v2 = ldf(vb + (size_t)rowbase[jj + 2] * p.Dv);
-        const float v3 = ldf(vb + (size_t)rowbase[jj + 3] * p.Dv);
+      // values of 8 consecutive keys are one vector (pieces start at multiples of 64 keys and
+      // blocks hold a multiple of 8): [..][key / 8][dv][key % 8]
+      for (int jj = 0; jj < nk; jj += 8) {
+        const int rb = rowbase[jj];                   // (blk G) BS + key offset in the block
+        const int blkG = rb / p.BS, off = rb - blkG * p.BS;
+        const T* vp = (const T*)p.v_cache +
+                      ((((size_t)(blkG + c) * (p.BS >> 3) + (off >> 3)) * p.Dv) + dv) * 8;
+        float v8[8];
+        ld8(vp, v8);
 #pragma unroll
         for (int g = 0; g < HMAX; ++g) {
           if (g < p.H) {
-            const float4 w4 = *(const float4*)(ps + g * TA_PIECE + jj);
-            acc[g] = fmaf(w4.x, v0, acc[g]);
-            acc[g] = fmaf(w4.y, v1, acc[g]);
-            acc[g] = fmaf(w4.z, v2, acc[g]);
-            acc[g] = fmaf(w4.w, v3, acc[g]);
+            const float4 w0 = *(const float4*)(ps + g * TA_PIECE + jj);
+            const float4 w1 = *(const float4*)(ps + g * TA_PIECE + jj + 4);
+            float a = acc[g];
+            a = fmaf(w0.x, v8[0], a);
+            a = fmaf(w0.y, v8[1], a);
+            a = fmaf(w0.z, v8[2], a);
+            a = fmaf(w0.w, v8[3], a);
+            a = fmaf(w1.x, v8[4], a);
+            a = fmaf(w1.y, v8[5], a);
+            a = fmaf(w1.z, v8[6], a);
+            a = fmaf(w1.w, v8[7], a);
+            acc[g] = a;
           }
         }
-      }
-      for (; jj < nk; ++jj) {
-        const float v0 = ldf(vb + (size_t)rowbase[jj] * p.Dv);
-#pragma unroll
-        for (int g = 0; g < HMAX; ++g)
-          if (g < p.H) acc[g] = fmaf(ps[g * TA_PIECE + jj], v0, acc[g]);
       }
     }
     __syncthreads();
@@ -426,7 +457,7 @@ __global__ __launch_bounds__(1024) void talking_merge_kernel(TalkParams p) {
   extern __shared__ float lds[];
   float* wgt = lds;                  // [parts][H] weight of a partition's sums
   float* inv_l = wgt + p.num_parts * p.H;
-  const int t = blockIdx.x;
+  const int t = blockIdx.x + p.row0;
   const int b = p.q_start ? find_seq(p.q_start, p.B, t) : t;
   if (p.seq_lens[b] <= 0) return;
   const int tid = threadIdx.x, nt = blockDim.x;
@@ -616,6 +647,22 @@ void launch_talking_attention(const TalkParams& p, bool f32, hipStream_t s) {
     if (p.H <= 8) AKAP_TA(bf16, 8); else if (p.H <= 16) AKAP_TA(bf16, 16); else AKAP_TA(bf16, 32);
   }
 #undef AKAP_TA
+}
+
+// the second launch alone, over rows [row0, T): normalise, mix the heads and gate what the
+// matrix-core kernel (or the split row kernel) left in the workspace
+void launch_talking_merge(const TalkParams& p, bool f32, hipStream_t s) {
+  const int rows = p.T - p.row0;
+  if (rows <= 0) return;
+  const int nt = ((p.G * p.Dv + 63) / 64) * 64;
+  const size_t mlds = (size_t)(p.num_parts + 1) * p.H * sizeof(float);
+#define AKAP_TM(TY, HM) talking_merge_kernel<TY, HM><<<rows, nt, mlds, s>>>(p)
+  if (f32) {
+    if (p.H <= 8) AKAP_TM(float, 8); else if (p.H <= 16) AKAP_TM(float, 16); else AKAP_TM(float, 32);
+  } else {
+    if (p.H <= 8) AKAP_TM(bf16, 8); else if (p.H <= 16) AKAP_TM(bf16, 16); else AKAP_TM(bf16, 32);
+  }
+#undef AKAP_TM
 }
 
 void launch_route_topk(int32_t* ids, float* w, const void* h, int h_stride, const float* router,

@@ -175,7 +175,7 @@ struct HeadNormParams {
   int proj_stride;
   void* q_out;        // [T, H, D]
   void* k_cache;      // [NB, G, BS, D]
-  void* v_cache;      // [NB, G, BS, Dv]
+  void* v_cache;      // [NB, G, BS / 8, Dv, 8]
   const int64_t* slots;
   int T, H, G, D, Dv, BS, q_off, k_off, v_off;
   int64_t num_slots;  // NB * BS
@@ -211,7 +211,7 @@ struct TalkParams {
   int out_stride;
   const void* q;        // [T, H, D]
   const void* k_cache;  // [NB, G, BS, D]
-  const void* v_cache;  // [NB, G, BS, Dv]
+  const void* v_cache;  // [NB, G, BS / 8, Dv, 8]
   const int32_t* block_tables;  // [B, max_blocks]
   int max_blocks;
   const int32_t* seq_lens;      // [B]
@@ -226,9 +226,18 @@ struct TalkParams {
   float* ws_ml;
   float* ws_o;
   int num_parts;
+  int row0;             // first row of a merge-only launch
 };
 size_t talking_attention_lds(int H, int D);
 void launch_talking_attention(const TalkParams& p, bool f32, hipStream_t s);
+void launch_talking_merge(const TalkParams& p, bool f32, hipStream_t s);
+// matrix-core form for prompt chunks (bf16): fills the workspace of a one-partition split for
+// the rows of the tile map (tile_seq / tile_row: sequence and first chunk row of a tile of
+// tile_rows tokens, a multiple of 32); launch_talking_merge finishes
+bool talk_mfma_supported(int H, int G, int D, int Dv, int BS);
+void launch_talking_prefill_mfma(const TalkParams& p, const int32_t* tile_seq,
+                                 const int32_t* tile_row, int num_tiles, int tile_rows,
+                                 hipStream_t s);
 
 void launch_route_topk(int32_t* ids, float* w, const void* h, int h_stride, const float* router,
                        const float* bias, int rows, int d, int n, int top, bool f32,

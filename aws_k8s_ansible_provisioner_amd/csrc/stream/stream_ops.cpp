@@ -740,10 +740,11 @@ void head_norm_cache(Tensor proj, Tensor q_out, Tensor k_cache, Tensor v_cache, 
                   v_off >= 0 && q_off + H * D <= N && k_off + G * D <= N && v_off + G * Dv <= N,
               "head_norm_cache: slices outside the projection");
   TORCH_CHECK(q_out.numel() == T * H * D && slots.numel() == T, "head_norm_cache: q_out / slots");
-  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.size(1) == G &&
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 5 && k_cache.size(1) == G &&
                   k_cache.size(3) == D && v_cache.size(0) == k_cache.size(0) &&
-                  v_cache.size(1) == G && v_cache.size(2) == k_cache.size(2) &&
-                  v_cache.size(3) == Dv, "head_norm_cache: cache shapes");
+                  v_cache.size(1) == G && v_cache.size(2) * 8 == k_cache.size(2) &&
+                  v_cache.size(3) == Dv && v_cache.size(4) == 8,
+              "head_norm_cache: K [NB, G, BS, D], V [NB, G, BS / 8, Dv, 8]");
   akap_stream::HeadNormParams p;
   p.proj = proj.data_ptr(); p.proj_stride = proj.stride(0);
   p.q_out = q_out.data_ptr(); p.k_cache = k_cache.data_ptr(); p.v_cache = v_cache.data_ptr();
@@ -808,22 +809,24 @@ void retention(Tensor out, Tensor proj, int64_t q_off, int64_t k_off, int64_t v_
   akap_stream::launch_retention(p, f32, cur_stream());
 }
 
-void talking_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables,
-                       Tensor seq_lens, std::optional<Tensor> q_start, Tensor positions,
-                       std::optional<Tensor> talk, std::optional<Tensor> gate, double scale,
-                       std::optional<Tensor> ws_ml, std::optional<Tensor> ws_o, int64_t num_parts) {
+// shared argument checks of the head-mixed attention ops; fills everything but the workspace
+akap_stream::TalkParams talk_params(const Tensor& out, const Tensor& q, const Tensor& k_cache,
+                                    const Tensor& v_cache, const Tensor& block_tables,
+                                    const Tensor& seq_lens, const std::optional<Tensor>& q_start,
+                                    const Tensor& positions, const std::optional<Tensor>& talk,
+                                    const std::optional<Tensor>& gate, double scale) {
   CHECK_GPU(out); CHECK_GPU(q); CHECK_GPU(k_cache); CHECK_GPU(v_cache); CHECK_GPU(block_tables);
   CHECK_GPU(seq_lens); CHECK_GPU(positions);
   CHECK_LAST_CONTIG(out); CHECK_CONTIG(q); CHECK_CONTIG(k_cache); CHECK_CONTIG(v_cache);
   CHECK_CONTIG(seq_lens); CHECK_CONTIG(positions);
-  const bool f32 = is_f32(q, "q");
   TORCH_CHECK(out.scalar_type() == q.scalar_type() && k_cache.scalar_type() == q.scalar_type() &&
                   v_cache.scalar_type() == q.scalar_type(), "talking_attention: dtypes differ");
-  TORCH_CHECK(q.dim() == 3 && k_cache.dim() == 4 && v_cache.dim() == 4, "talking_attention: ranks");
+  TORCH_CHECK(q.dim() == 3 && k_cache.dim() == 4 && v_cache.dim() == 5, "talking_attention: ranks");
   const int64_t T = q.size(0), H = q.size(1), D = q.size(2);
   const int64_t G = k_cache.size(1), BS = k_cache.size(2), Dv = v_cache.size(3);
   TORCH_CHECK(k_cache.size(3) == D && v_cache.size(0) == k_cache.size(0) && v_cache.size(1) == G &&
-                  v_cache.size(2) == BS && G > 0 && H % G == 0, "talking_attention: cache shapes");
+                  v_cache.size(2) * 8 == BS && v_cache.size(4) == 8 && G > 0 && H % G == 0,
+              "talking_attention: K [NB, G, BS, D], V [NB, G, BS / 8, Dv, 8]");
   TORCH_CHECK(H <= 32 && G * Dv <= 1024,
               "talking_attention: at most 32 heads and 1024 value entries per token");
   TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) >= H * Dv, "talking_attention: out");
@@ -865,20 +868,62 @@ void talking_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache, Ten
   }
   p.scale = (float)scale;
   p.T = T; p.H = H; p.G = G; p.D = D; p.Dv = Dv; p.BS = BS;
-  p.ws_ml = nullptr; p.ws_o = nullptr; p.num_parts = 1;
-  if (num_parts > 1) {
-    TORCH_CHECK(ws_ml.has_value() && ws_o.has_value(), "talking_attention: a workspace for parts");
-    CHECK_GPU(*ws_ml); CHECK_GPU(*ws_o); CHECK_F32(*ws_ml); CHECK_F32(*ws_o);
-    TORCH_CHECK(ws_ml->numel() >= T * num_parts * H * 2 &&
-                    ws_o->numel() >= T * num_parts * H * G * Dv, "talking_attention: workspace size");
-    p.ws_ml = ws_ml->data_ptr<float>(); p.ws_o = ws_o->data_ptr<float>();
-    p.num_parts = num_parts;
-    TORCH_CHECK((num_parts + 1) * H * 4 <= 65536, "talking_attention: too many partitions");
-  }
+  p.ws_ml = nullptr; p.ws_o = nullptr; p.num_parts = 1; p.row0 = 0;
   TORCH_CHECK(akap_stream::talking_attention_lds(H, D) <= 65536,
               "talking_attention: heads x head size too large for the query row in LDS");
+  return p;
+}
+
+void talk_workspace(akap_stream::TalkParams& p, const std::optional<Tensor>& ws_ml,
+                    const std::optional<Tensor>& ws_o, int64_t num_parts) {
+  TORCH_CHECK(ws_ml.has_value() && ws_o.has_value(), "talking_attention: a workspace is needed");
+  CHECK_GPU(*ws_ml); CHECK_GPU(*ws_o); CHECK_F32(*ws_ml); CHECK_F32(*ws_o);
+  TORCH_CHECK(ws_ml->numel() >= (int64_t)p.T * num_parts * p.H * 2 &&
+                  ws_o->numel() >= (int64_t)p.T * num_parts * p.H * p.G * p.Dv,
+              "talking_attention: workspace size");
+  TORCH_CHECK((num_parts + 1) * p.H * 4 <= 65536, "talking_attention: too many partitions");
+  p.ws_ml = ws_ml->data_ptr<float>(); p.ws_o = ws_o->data_ptr<float>();
+  p.num_parts = num_parts;
+}
+
+void talking_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables,
+                       Tensor seq_lens, std::optional<Tensor> q_start, Tensor positions,
+                       std::optional<Tensor> talk, std::optional<Tensor> gate, double scale,
+                       std::optional<Tensor> ws_ml, std::optional<Tensor> ws_o, int64_t num_parts) {
+  akap_stream::TalkParams p = talk_params(out, q, k_cache, v_cache, block_tables, seq_lens, q_start,
+                                          positions, talk, gate, scale);
+  if (num_parts > 1) talk_workspace(p, ws_ml, ws_o, num_parts);
   const c10::DeviceGuard g(q.device());
-  akap_stream::launch_talking_attention(p, f32, cur_stream());
+  akap_stream::launch_talking_attention(p, is_f32(q, "q"), cur_stream());
+}
+
+bool talking_mfma_supported(int64_t H, int64_t G, int64_t D, int64_t Dv, int64_t BS) {
+  return akap_stream::talk_mfma_supported((int)H, (int)G, (int)D, (int)Dv, (int)BS);
+}
+
+void talking_attention_prefill_mfma(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
+                                    Tensor block_tables, Tensor seq_lens, Tensor q_start,
+                                    Tensor positions, Tensor tile_seq, Tensor tile_row,
+                                    int64_t tile_rows, int64_t first_row,
+                                    std::optional<Tensor> talk, std::optional<Tensor> gate,
+                                    double scale, Tensor ws_ml, Tensor ws_o) {
+  akap_stream::TalkParams p = talk_params(out, q, k_cache, v_cache, block_tables, seq_lens, q_start,
+                                          positions, talk, gate, scale);
+  TORCH_CHECK(q.scalar_type() == at::kBFloat16 &&
+                  akap_stream::talk_mfma_supported(p.H, p.G, p.D, p.Dv, p.BS),
+              "talking_attention_prefill_mfma: bf16 and sizes the matrix-core kernel takes");
+  talk_workspace(p, ws_ml, ws_o, 1);
+  CHECK_GPU(tile_seq); CHECK_GPU(tile_row); CHECK_CONTIG(tile_seq); CHECK_CONTIG(tile_row);
+  TORCH_CHECK(tile_seq.scalar_type() == at::kInt && tile_row.scalar_type() == at::kInt &&
+                  tile_row.numel() >= tile_seq.numel() && tile_rows >= 32 && tile_rows % 32 == 0,
+              "talking_attention_prefill_mfma: tile map");
+  TORCH_CHECK(first_row >= 0 && first_row <= p.T, "talking_attention_prefill_mfma: first_row");
+  p.row0 = first_row;
+  const c10::DeviceGuard g(q.device());
+  akap_stream::launch_talking_prefill_mfma(p, tile_seq.data_ptr<int32_t>(),
+                                           tile_row.data_ptr<int32_t>(), (int)tile_seq.numel(),
+                                           (int)tile_rows, cur_stream());
+  akap_stream::launch_talking_merge(p, false, cur_stream());
 }
 
 void route_topk(Tensor ids, Tensor w, Tensor h, Tensor router, std::optional<Tensor> bias) {
@@ -983,6 +1028,12 @@ TORCH_LIBRARY(akap_stream, m) {
   m.def("talking_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, "
         "Tensor block_tables, Tensor seq_lens, Tensor? q_start, Tensor positions, Tensor? talk, "
         "Tensor? gate, float scale, Tensor(b!)? ws_ml, Tensor(c!)? ws_o, int num_parts) -> ()");
+  m.def("talking_mfma_supported(int H, int G, int D, int Dv, int BS) -> bool",
+        &talking_mfma_supported);
+  m.def("talking_attention_prefill_mfma(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, "
+        "Tensor block_tables, Tensor seq_lens, Tensor q_start, Tensor positions, Tensor tile_seq, "
+        "Tensor tile_row, int tile_rows, int first_row, Tensor? talk, Tensor? gate, float scale, "
+        "Tensor(b!) ws_ml, Tensor(c!) ws_o) -> ()");
   m.def("route_topk(Tensor(a!) ids, Tensor(b!) w, Tensor h, Tensor router, Tensor? bias) -> ()");
   m.def("swiglu_routed(Tensor(a!) out, Tensor gu, Tensor? ids, Tensor? w, int experts) -> ()");
 }
@@ -1005,6 +1056,7 @@ TORCH_LIBRARY_IMPL(akap_stream, CUDA, m) {
   m.impl("head_norm_cache", &head_norm_cache);
   m.impl("retention", &retention);
   m.impl("talking_attention", &talking_attention);
+  m.impl("talking_attention_prefill_mfma", &talking_attention_prefill_mfma);
   m.impl("route_topk", &route_topk);
   m.impl("swiglu_routed", &swiglu_routed);
   m.impl("embed_scaled", &embed_scaled);

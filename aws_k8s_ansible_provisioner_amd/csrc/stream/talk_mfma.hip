@@ -1,0 +1,202 @@
+// Head-mixed attention of prompt chunks on the matrix cores (bf16 cache).
+//
+// One workgroup of four waves per (tile of 32 queries of one sequence, query head g).  Keys go
+// by steps of 128: wave w scores keys [32 w, 32 w + 32) of the step (S^T = K Q^T on
+// v_mfma_f32_32x32x16_bf16: a query is a lane column, so its running max and sum are per-lane
+// values plus one exchange between the lane halves; the K rows are taken in an order -- bits 2
+// and 3 of the row swapped -- that makes a lane's accumulator registers 8 consecutive keys,
+// i.e. an operand of the next product without lane traffic).  The waves agree on the step's
+// maximum through LDS and publish their bf16 weights there; then every wave accumulates, for
+// ITS share of the (value head, 32 value entries) column tiles, O = P V over all 128 keys of
+// the step (values come from the cache in groups of 8 keys, one 16-byte load per lane and
+// operand).  A workgroup thus forms, for its query head, the unnormalised sums of ALL value
+// heads; they go to a workspace (fp32) with the head's (max, sum), and the merge launch of the
+// split row kernel normalises, mixes the heads and gates.
+#include "../kernels/common.h"
+#include "stream.h"
+
+namespace akap_stream {
+
+using akap::bf16;
+using akap::bf16x8;
+using akap::f32x16;
+
+namespace {
+
+__device__ __forceinline__ int swap23(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1); }
+
+template <int TPW>
+__global__ __launch_bounds__(256) void talk_prefill_mfma_kernel(TalkParams p, const int32_t* tile_seq,
+                                                               const int32_t* tile_row,
+                                                               int tile_rows) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int KS = p.D >> 4;                         // 16-wide steps of the head size
+  bf16x8* qs = (bf16x8*)smem;                      // [KS][64] Q operands
+  bf16x8* ps = qs + KS * 64;                       // [2][4][2][64] weights of a step
+  float* m_loc = (float*)(ps + 2 * 4 * 2 * 64);    // [2][4][32] each wave's maxima
+  float* alpha_s = m_loc + 2 * 4 * 32;             // [2][32] rescale of the step
+  float* l_s = alpha_s + 2 * 32;                   // [4][32] the waves' sums at the end
+
+  const int sub_per = tile_rows >> 5;
+  const int tile = blockIdx.x / sub_per, sub = blockIdx.x - tile * sub_per;
+  const int g = blockIdx.y;
+  const int b = tile_seq[tile];
+  const int r_first = tile_row[tile] + 32 * sub;
+  const int chunk = p.q_start[b + 1] - p.q_start[b];
+  if (r_first >= chunk) return;
+  const int t0 = p.q_start[b] + r_first;
+  const int nrows = min(32, chunk - r_first);
+  const int pos0 = (int)p.positions[t0];
+  const int kmax = pos0 + nrows - 1;               // last key any query of the tile sees
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int col = lane & 31, hf = lane >> 5;
+  const int rep = p.H / p.G, kvh = g / rep;
+  const int32_t* bt = p.block_tables + (size_t)b * p.max_blocks;
+  const float sc2 = p.scale * 1.44269504088896f;   // scores -> log2 units
+  const int DVT = p.Dv >> 5, NT = p.G * DVT;       // column tiles of 32 value entries
+
+  // Q operands: lane (col = query, hf) of step c holds Q[t0 + col][16 c + 8 hf ..+8]
+  for (int e = tid; e < KS * 64; e += 256) {
+    const int c = e >> 6, ln = e & 63;
+    const int qc = ln & 31, qh = ln >> 5;
+    bf16x8 v;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (bf16)0.f;
+    if (qc < nrows)
+      v = *(const bf16x8*)((const bf16*)p.q + ((size_t)(t0 + qc) * p.H + g) * p.D + 16 * c + 8 * qh);
+    qs[e] = v;
+  }
+  f32x16 acc[TPW];
+#pragma unroll
+  for (int k = 0; k < TPW; ++k)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[k][i] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const int qpos = col < nrows ? pos0 + col : -1;  // -1: an unused column sees nothing
+  __syncthreads();
+
+  int buf = 0;
+  for (int key0 = 0; key0 <= kmax; key0 += 128, buf ^= 1) {
+    // ---- scores of my 32 keys
+    const int kb = key0 + 32 * wave;
+    f32x16 s;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+    if (kb <= kmax) {
+      const int key = min(kb + swap23(col), kmax);  // rows past the range are masked below
+      const int bi = key / p.BS;
+      const bf16* kp = (const bf16*)p.k_cache +
+                       ((size_t)(bt[bi] * p.G + kvh) * p.BS + (key - bi * p.BS)) * p.D + 8 * hf;
+      for (int c = 0; c < KS; ++c) {
+        const bf16x8 kf = *(const bf16x8*)(kp + 16 * c);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qs[c * 64 + lane], s, 0, 0, 0);
+      }
+    }
+    // register i of this lane: key kb + 16 (i >> 3) + 8 hf + (i & 7), query column col
+    float bmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int key = kb + 16 * (i >> 3) + 8 * hf + (i & 7);
+      s[i] = key <= qpos ? s[i] * sc2 : -INFINITY;
+      bmax = fmaxf(bmax, s[i]);
+    }
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+    if (hf == 0) m_loc[(buf * 4 + wave) * 32 + col] = bmax;
+    __syncthreads();
+    const float* ml = m_loc + buf * 4 * 32 + col;
+    const float mn = fmaxf(fmaxf(m_run, fmaxf(ml[0], ml[32])), fmaxf(ml[64], ml[96]));
+    const float ms = mn == -INFINITY ? 0.f : mn;    // nothing visible yet: every exp below is 0
+    const float alpha = __builtin_amdgcn_exp2f(m_run - ms);
+    m_run = mn;
+    float psum = 0.f;
+    bf16x8 pb[2];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float e = __builtin_amdgcn_exp2f(s[i] - ms);
+      psum += e;
+      pb[i >> 3][i & 7] = (bf16)e;
+    }
+    l_run = l_run * alpha + psum;
+    ps[((buf * 4 + wave) * 2 + 0) * 64 + lane] = pb[0];
+    ps[((buf * 4 + wave) * 2 + 1) * 64 + lane] = pb[1];
+    if (wave == 0 && hf == 0) alpha_s[buf * 32 + col] = alpha;
+    __syncthreads();
+    // ---- O += P V for my column tiles; accumulator register i: query row
+    //      (i & 3) + 4 hf + 8 ((i >> 2) & 1) + 16 (i >> 3), value entry col of the tile
+    float ar[16];
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const float4 a4 = *(const float4*)(alpha_s + buf * 32 + 4 * hf + 8 * (i4 & 1) + 16 * (i4 >> 1));
+      ar[4 * i4] = a4.x; ar[4 * i4 + 1] = a4.y; ar[4 * i4 + 2] = a4.z; ar[4 * i4 + 3] = a4.w;
+    }
+#pragma unroll
+    for (int k = 0; k < TPW; ++k) {
+      const int ti = wave + 4 * k;
+      if (ti < NT) {
+        const int cv = ti / DVT, dv0 = (ti - cv * DVT) << 5;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[k][i] *= ar[i];
+        for (int w2 = 0; w2 < 4; ++w2) {
+#pragma unroll
+          for (int sl = 0; sl < 2; ++sl) {
+            const int kg = key0 + 32 * w2 + 16 * sl;   // first key of this 16-key operand
+            if (kg <= kmax) {
+              const int kk = min(kg + 8 * hf, kmax);   // a group wholly past the range: weights 0
+              const int bi = kk / p.BS;
+              const int off = kk - bi * p.BS;
+              const bf16* vp = (const bf16*)p.v_cache +
+                               ((((size_t)(bt[bi] * p.G + cv) * (p.BS >> 3) + (off >> 3)) * p.Dv) +
+                                dv0 + col) * 8;
+              const bf16x8 vf = *(const bf16x8*)vp;
+              acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                  ps[((buf * 4 + w2) * 2 + sl) * 64 + lane], vf, acc[k], 0, 0, 0);
+            }
+          }
+        }
+      }
+    }
+  }
+  // ---- the head's (max, sum) and its unnormalised sums
+  l_run += __shfl_xor(l_run, 32, 64);
+  if (hf == 0) l_s[wave * 32 + col] = l_run;
+  __syncthreads();
+  if (wave == 0 && hf == 0 && col < nrows) {
+    const size_t cell = ((size_t)(t0 + col) * p.H + g) * 2;
+    p.ws_ml[cell] = m_run * 0.6931471805599453f;
+    p.ws_ml[cell + 1] = l_s[col] + l_s[32 + col] + l_s[64 + col] + l_s[96 + col];
+  }
+  const int GV = p.G * p.Dv;
+#pragma unroll
+  for (int k = 0; k < TPW; ++k) {
+    const int ti = wave + 4 * k;
+    if (ti < NT) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int row = (i & 3) + 4 * hf + 8 * ((i >> 2) & 1) + 16 * (i >> 3);
+        if (row < nrows)
+          p.ws_o[((size_t)(t0 + row) * p.H + g) * GV + (ti << 5) + col] = acc[k][i];
+      }
+    }
+  }
+}
+
+}  // namespace
+
+bool talk_mfma_supported(int H, int G, int D, int Dv, int BS) {
+  return H <= 32 && D % 16 == 0 && D <= 256 && Dv % 32 == 0 && G * (Dv / 32) <= 32 && BS % 16 == 0;
+}
+
+void launch_talking_prefill_mfma(const TalkParams& p, const int32_t* tile_seq,
+                                 const int32_t* tile_row, int num_tiles, int tile_rows,
+                                 hipStream_t s) {
+  if (num_tiles <= 0) return;
+  const int NT = p.G * (p.Dv / 32);
+  const dim3 grid(num_tiles * (tile_rows / 32), p.H);
+  const size_t lds = (size_t)(p.D / 16) * 64 * 16 + 2 * 4 * 2 * 64 * 16 +
+                     (2 * 4 * 32 + 2 * 32 + 4 * 32) * sizeof(float);
+  if (NT <= 8) talk_prefill_mfma_kernel<2><<<grid, 256, lds, s>>>(p, tile_seq, tile_row, tile_rows);
+  else if (NT <= 16) talk_prefill_mfma_kernel<4><<<grid, 256, lds, s>>>(p, tile_seq, tile_row, tile_rows);
+  else talk_prefill_mfma_kernel<8><<<grid, 256, lds, s>>>(p, tile_seq, tile_row, tile_rows);
+}
+
+}  // namespace akap_stream

@@ -274,11 +274,15 @@ class SazepelLM:
 
     def allocate_kv_segments(self, num_blocks: int, block_size: int, kv_dtype: str = "auto",
                              max_segment_bytes: Optional[int] = None) -> list:
-        """Per layer run with an attention: K [NB, G, BS, D] and V [NB, G, BS, Dv], token-major,
-        zero-filled, in the model's dtype.  Retention layers cache nothing per token (a model
+        """Per layer run with an attention: K [NB, G, BS, D] (token-major rows) and V
+        [NB, G, BS / 8, Dv, 8] (groups of 8 tokens, dimension-major inside a group: the 8 keys a
+        matrix-core operand contracts over, or a decode lane accumulates, are one 16-byte
+        load), zero-filled, in the model's dtype.  Retention layers cache nothing per token (a model
         of retention layers only gets one placeholder so the pool has a dtype)."""
         if kv_dtype not in ("auto", "bf16", "bfloat16"):
             raise ValueError("Sazepel: the KV cache is kept in the model's dtype (no fp8)")
+        if block_size % 8:
+            raise ValueError("Sazepel: the block size must be a multiple of 8")
         segs, self._seg_map = [], {}
         for r, i in enumerate(self.runs):
             a, _ = self._parts(self.cfg.layer_specs[i])
@@ -287,8 +291,8 @@ class SazepelLM:
             self._seg_map[r] = len(segs)
             segs.append(torch.zeros(num_blocks, a.kv_heads, block_size, a.dim, dtype=self.dtype,
                                     device=self.device))
-            segs.append(torch.zeros(num_blocks, a.kv_heads, block_size, a.vdim, dtype=self.dtype,
-                                    device=self.device))
+            segs.append(torch.zeros(num_blocks, a.kv_heads, block_size // 8, a.vdim, 8,
+                                    dtype=self.dtype, device=self.device))
         if not segs:
             segs.append(torch.zeros(1, dtype=self.dtype, device=self.device))
         return segs
@@ -346,8 +350,10 @@ class SazepelLM:
         gate = proj[:, nq + nk + nv:nq + nk + nv + a.heads * a.vdim] if a.gate else None
         talk = lw.talk if a.talk else None
         if batch.is_prefill:
-            sops.talking_attention(out, q, kc, vc, batch.block_tables, batch.seq_lens,
-                                   batch.q_start, batch.positions, talk, gate, a.scale)
+            sops.talking_attention_prefill(out, q, kc, vc, batch.block_tables, batch.seq_lens,
+                                           batch.q_start, batch.positions, batch.tile_seq,
+                                           batch.tile_row, batch.tile_rows, talk, gate, a.scale,
+                                           first_seq=batch.num_decode)
             return
         parts, ws = 1, None
         if q.is_cuda:

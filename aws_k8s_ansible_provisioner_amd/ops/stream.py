@@ -672,8 +672,8 @@ def head_norm_cache(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tens
                     norm_v: bool = True) -> None:
     """Per token t of the fused projection proj [T, N]: the H query heads
     proj[t, q_off : q_off + H D] go to q_out [T, H, D], the G key heads (from k_off) to k_cache
-    [NB, G, BS, D] and the G value heads (from v_off, size Dv) to v_cache [NB, G, BS, Dv] at
-    slots[t] (-1: nothing is cached).  norm_qk / norm_v: each head is first divided by its own
+    [NB, G, BS, D] and the G value heads (from v_off, size Dv) to v_cache [NB, G, BS / 8, Dv, 8]
+    (groups of 8 tokens, dimension-major inside a group) at slots[t] (-1: nothing is cached).  norm_qk / norm_v: each head is first divided by its own
     root mean square (fp32, eps inside the root, no weights)."""
     if _native(proj):
         torch.ops.akap_stream.head_norm_cache(proj, q_out, k_cache, v_cache, slots, H, G, D, Dv,
@@ -693,7 +693,7 @@ def head_norm_cache(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tens
     ok = slots >= 0
     sl = slots[ok].long()
     k_cache[sl // BS, :, sl % BS] = k[ok].to(k_cache.dtype)
-    v_cache[sl // BS, :, sl % BS] = v[ok].to(v_cache.dtype)
+    v_cache[sl // BS, :, (sl % BS) // 8, :, sl % 8] = v[ok].to(v_cache.dtype)
 
 
 def talking_attention_parts(rows: int, kv_heads: int, max_len: int) -> int:
@@ -724,7 +724,7 @@ def talking_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
     sigmoid(gate[t, h Dv + i]) per entry when gate is given.  talk None: no mixing.
     Row t belongs to sequence b with q_start[b] <= t < q_start[b + 1] (q_start None: row t is
     sequence t); sequences with seq_lens[b] == 0 are padding and their rows are left unwritten.
-    q [T, H, D]; k_cache [NB, G, BS, D]; v_cache [NB, G, BS, Dv]; talk fp32 [H, H]; gate and
+    q [T, H, D]; k_cache [NB, G, BS, D]; v_cache [NB, G, BS / 8, Dv, 8]; talk fp32 [H, H]; gate and
     out are [T, H Dv] views that may be column slices of wider rows.  Scores, softmax, the
     mixing and the gate are fp32.
     The GPU kernel forms, for every head g, the unnormalised sums of ALL G value heads under
@@ -740,8 +740,8 @@ def talking_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
     T, H, D = q.shape
     G, BS, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
     rep = H // G
-    B = seq_lens.numel()
-    for b in range(B):
+    B = seq_lens.numel() if q_start is None else min(seq_lens.numel(), q_start.numel() - 1)
+    for b in range(min(B, T) if q_start is None else B):
         kv = int(seq_lens[b])
         r0, r1 = (b, b + 1) if q_start is None else (int(q_start[b]), int(q_start[b + 1]))
         if kv == 0 or r1 <= r0:
@@ -749,7 +749,7 @@ def talking_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
         nb = -(-kv // BS)
         blocks = block_tables[b, :nb].long()
         K = k_cache[blocks].permute(1, 0, 2, 3).reshape(G, nb * BS, D)[:, :kv].float()
-        V = v_cache[blocks].permute(1, 0, 2, 3).reshape(G, nb * BS, Dv)[:, :kv].float()
+        V = v_tokens(v_cache[blocks]).permute(1, 0, 2, 3).reshape(G, nb * BS, Dv)[:, :kv].float()
         pos = positions[r0:r1].long()
         ok = torch.arange(kv)[None, :] <= pos[:, None]
         s = torch.einsum("thd,hjd->htj", q[r0:r1].float(), K.repeat_interleave(rep, dim=0)) * scale
@@ -760,6 +760,40 @@ def talking_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
         if gate is not None:
             o = o * torch.sigmoid(gate[r0:r1].float())
         out[r0:r1] = o.to(out.dtype)
+
+
+def talking_attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
+                              v_cache: torch.Tensor, block_tables: torch.Tensor,
+                              seq_lens: torch.Tensor, q_start: torch.Tensor,
+                              positions: torch.Tensor, tile_seq, tile_row, tile_rows: int,
+                              talk: Optional[torch.Tensor], gate: Optional[torch.Tensor],
+                              scale: float, first_seq: int = 0) -> None:
+    """talking_attention for a step with prompt chunks.  The rows of the sequences before
+    first_seq (single-token sequences that lead a mixed step, one row each) go through the row
+    kernel; the chunks, on the GPU in bf16 and at sizes the matrix-core kernel takes, run on
+    the matrix cores, driven by the scheduler's tile map (tile_seq / tile_row: sequence and
+    first chunk row of a tile of tile_rows tokens): per query head the unnormalised sums of all
+    value heads, then one launch that normalises, mixes the heads and gates."""
+    H, D = q.shape[1], q.shape[2]
+    G, BS, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    T = q.shape[0]
+    if (q.is_cuda and q.dtype == torch.bfloat16 and tile_seq is not None and tile_rows % 32 == 0
+            and load_native(required=True)
+            and torch.ops.akap_stream.talking_mfma_supported(H, G, D, Dv, BS)):
+        nd = first_seq
+        if nd:
+            talking_attention(out[:nd], q[:nd], k_cache, v_cache, block_tables[:nd], seq_lens[:nd],
+                              None, positions[:nd], talk, gate[:nd] if gate is not None else None,
+                              scale)
+        if T > nd:
+            ws_ml = torch.empty(T * H * 2, dtype=torch.float32, device=q.device)
+            ws_o = torch.empty(T * H * G * Dv, dtype=torch.float32, device=q.device)
+            torch.ops.akap_stream.talking_attention_prefill_mfma(
+                out, q, k_cache, v_cache, block_tables, seq_lens, q_start, positions, tile_seq,
+                tile_row, int(tile_rows), int(nd), talk, gate, float(scale), ws_ml, ws_o)
+        return
+    talking_attention(out, q, k_cache, v_cache, block_tables, seq_lens, q_start, positions, talk,
+                      gate, scale)
 
 
 # ----------------------------------------------------------------------------- retention

@@ -234,7 +234,9 @@ def _attention_case(seed, lens, rows, H, G, D, V, BS, talk=True):
     T = sum(rows)
     q = torch.randn(T, H, D, generator=g)
     tk = torch.randn(H, H, generator=g) if talk else None
-    return dict(q=q, ks=ks, vs=vs, kc=kc, vc=vc, bt=bt, talk=tk, lens=lens, rows=rows)
+    # the value cache keeps groups of 8 tokens, dimension-major inside a group
+    return dict(q=q, ks=ks, vs=vs, kc=kc, vc=sops.v_from_tokens(vc), bt=bt, talk=tk, lens=lens,
+                rows=rows)
 
 
 def _attention_run(c, scale, gate=None):
@@ -286,7 +288,7 @@ def test_attention_sees_one_dominant_key(far):
             c["q"][row] = c["ks"][0][far, 0]      # both heads ask for it
     got = _attention_run(c, 1.0).to(F64)
     torch.testing.assert_close(got, _attention_want(c, 1.0), rtol=1e-4, atol=1e-4)
-    torch.testing.assert_close(got[39, :4], c["vc"][blk, 0, far % 32].to(F64), rtol=0.05, atol=0.05)
+    torch.testing.assert_close(got[39, :4], c["vs"][0][far, 0].to(F64), rtol=0.05, atol=0.05)
 
 
 def test_attention_does_not_see_the_future():
@@ -302,7 +304,8 @@ def test_per_head_norms_and_cached_values():
     proj = torch.randn(T, H * D + G * D + G * V + 3, generator=g) * \
         torch.logspace(-2, 2, T)[:, None]                              # rows of very different size
     q = torch.zeros(T, H, D)
-    kc, vc = torch.zeros(5, G, BS, D), torch.zeros(5, G, BS, V)
+    T, H, G, D, V, BS, eps = 7, 4, 2, 6, 10, 8, 1e-3
+    kc, vc = torch.zeros(5, G, BS, D), torch.zeros(5, G, BS // 8, V, 8)
     slots = torch.tensor([8, 9, 10, 11, 3, -1, 17])
     sops.head_norm_cache(proj, q, kc, vc, slots, H, G, D, V, 1, 1 + H * D, 1 + (H + G) * D, eps)
     p = proj.to(F64)
@@ -313,7 +316,8 @@ def test_per_head_norms_and_cached_values():
     for t, s in enumerate(slots.tolist()):
         if s >= 0:
             torch.testing.assert_close(kc[s // BS, :, s % BS].to(F64), wk[t], rtol=1e-5, atol=1e-5)
-            torch.testing.assert_close(vc[s // BS, :, s % BS].to(F64), wv[t], rtol=1e-5, atol=1e-5)
+            torch.testing.assert_close(sops.v_tokens(vc)[s // BS, :, s % BS].to(F64), wv[t],
+                                       rtol=1e-5, atol=1e-5)
     assert kc.abs().sum(dim=(1, 3)).flatten().count_nonzero() == 6     # the padding row wrote nothing
 
 

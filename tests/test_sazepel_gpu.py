@@ -65,7 +65,7 @@ def test_head_norm_cache_kernel(dtype, H, G, D, Dv):
         for nq, nv in ((True, True), (False, True), (True, False)):
             q = torch.zeros(T, H, D, dtype=dt, device=dev)
             kc = torch.zeros(NB, G, BS, D, dtype=dt, device=dev)
-            vc = torch.zeros(NB, G, BS, Dv, dtype=dt, device=dev)
+            vc = torch.zeros(NB, G, BS // 8, Dv, 8, dtype=dt, device=dev)
             sops.head_norm_cache(proj.to(dev), q, kc, vc, slots.to(dev), H, G, D, Dv, 3, 3 + H * D,
                                  3 + H * D + G * D, 1e-6, nq, nv)
             res.append((q, kc, vc))
@@ -121,7 +121,7 @@ def _attention_case(dtype, H, G, D, Dv, dev, g, parts, talk=True, gate=True, BS=
     rows = [5, 1, 33, 1]                        # rows of this step (the last positions)
     NB = sum(-(-n // BS) for n in lens) + 2
     kc = torch.randn(NB, G, BS, D, generator=g).to(dt)
-    vc = torch.randn(NB, G, BS, Dv, generator=g).to(dt)
+    vc = torch.randn(NB, G, BS // 8, Dv, 8, generator=g).to(dt)
     perm = torch.randperm(NB, generator=g).int()
     mb = max(-(-n // BS) for n in lens)
     bt = torch.zeros(len(lens), mb, dtype=torch.int32)
@@ -163,7 +163,7 @@ def test_talking_attention_decode_rows_without_sequence_starts():
     H, G, D, Dv, BS = 4, 2, 32, 16, 32
     lens = torch.tensor([40, 0, 200, 1], dtype=torch.int32)
     NB = 12
-    kc, vc = torch.randn(NB, G, BS, D, generator=g), torch.randn(NB, G, BS, Dv, generator=g)
+    kc, vc = torch.randn(NB, G, BS, D, generator=g), torch.randn(NB, G, BS // 8, Dv, 8, generator=g)
     bt = torch.tensor([[0, 1, 0, 0, 0, 0, 0], [0] * 7, [2, 3, 4, 5, 6, 7, 8], [9, 0, 0, 0, 0, 0, 0]],
                       dtype=torch.int32)
     q = torch.randn(4, H, D, generator=g)
@@ -179,6 +179,55 @@ def test_talking_attention_decode_rows_without_sequence_starts():
     assert (outs[0][1] == 7.0).all() and (outs[1][1] == 7.0).all() and (outs[2][1] == 7.0).all()
     close(outs[1], outs[0], "float32")
     close(outs[2], outs[0], "float32")
+
+
+def _tile_map(q_start, first_seq, tile_rows):
+    """The scheduler's prefill tile map: (sequence, first chunk row) per tile of tile_rows."""
+    seqs, rows = [], []
+    for b in range(first_seq, len(q_start) - 1):
+        for r in range(0, q_start[b + 1] - q_start[b], tile_rows):
+            seqs.append(b)
+            rows.append(r)
+    return (torch.tensor(seqs, dtype=torch.int32, device="cuda"),
+            torch.tensor(rows, dtype=torch.int32, device="cuda"))
+
+
+@pytest.mark.parametrize("H,G,D,Dv,BS", [(6, 3, 96, 96, 32), (4, 1, 16, 32, 16), (8, 8, 32, 64, 32),
+                                         (16, 4, 128, 128, 32), (2, 2, 48, 160, 16),
+                                         (32, 8, 64, 128, 32)])
+def test_talking_attention_matrix_core_kernel(H, G, D, Dv, BS):
+    """Prompt chunks on the matrix cores against the op on the CPU: chunks that start at 0 and
+    in the middle of a sequence, tiles cut by a chunk's end, single rows that lead the step."""
+    g = gen(H + D)
+    lens = [9, 301, 140, 33, 700]               # cached keys per sequence after this step
+    rows = [1, 1, 140, 20, 333]                 # two single-token sequences lead
+    NB = sum(-(-n // BS) for n in lens) + 2
+    kc = torch.randn(NB, G, BS, D, generator=g).bfloat16()
+    vc = torch.randn(NB, G, BS // 8, Dv, 8, generator=g).bfloat16()
+    perm = torch.randperm(NB, generator=g).int()
+    bt = torch.zeros(len(lens), max(-(-n // BS) for n in lens), dtype=torch.int32)
+    o = 0
+    for b, n in enumerate(lens):
+        nb = -(-n // BS)
+        bt[b, :nb] = perm[o:o + nb]
+        o += nb
+    T = sum(rows)
+    q = (0.5 * torch.randn(T, H, D, generator=g)).bfloat16()
+    pos = torch.cat([torch.arange(n - r, n) for n, r in zip(lens, rows)])
+    qs = torch.tensor([0] + rows, dtype=torch.int32).cumsum(0).int()
+    tk = torch.eye(H) + 0.3 * torch.randn(H, H, generator=g)
+    gt = torch.randn(T, H * Dv, generator=g).bfloat16()
+    sl = torch.tensor(lens, dtype=torch.int32)
+    want = torch.zeros(T, H * Dv, dtype=torch.bfloat16)
+    sops.talking_attention(want, q, kc, vc, bt, sl, qs, pos, tk, gt, 0.3)
+    for tile_rows in (128, 32):
+        ts, tr = _tile_map(qs.tolist(), 2, tile_rows)
+        out = torch.zeros(T, H * Dv + 8, dtype=torch.bfloat16, device="cuda")
+        sops.talking_attention_prefill(out[:, :H * Dv], q.cuda(), kc.cuda(), vc.cuda(), bt.cuda(),
+                                       sl.cuda(), qs.cuda(), pos.cuda(), ts, tr, tile_rows,
+                                       tk.cuda(), gt.cuda(), 0.3, first_seq=2)
+        close(out[:, :H * Dv], want, "bfloat16")
+        assert (out[:, H * Dv:] == 0).all()
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
