@@ -153,7 +153,17 @@ __global__ __launch_bounds__(256) void head_norm_cache_kernel(HeadNormParams p) 
 // by lane exchange), then the outputs of the TC tokens are normed and gated, a wave per token.
 constexpr int RET_TC = 16;   // tokens staged at a time (8 when the rows of 16 exceed 64 KB)
 
-template <typename T, int DREG>
+// Long prompt chunks run in three launches over segments of p.SEG rows, so that a sequence's
+// segments proceed side by side: MODE 1 leaves each segment's own state (started from zeros, no
+// outputs) in seg_buf, retention_scan_kernel turns these into the state BEFORE each segment (and
+// the sequence's final state in its slot), MODE 3 produces the outputs of each segment from
+// that.  MODE 0 is the direct form: a workgroup walks all rows of its sequence.
+// Segment buffers are indexed compactly: sequence b owns entries from q_start[b] / SEG + b.
+__device__ __forceinline__ int seg_base(const int32_t* q_start, int b, int SEG) {
+  return q_start[b] / SEG + b;
+}
+
+template <typename T, int DREG, int MODE>
 __global__ __launch_bounds__(1024) void retention_kernel(RetentionParams p) {
   extern __shared__ float lds[];
   const int DP = p.DP;                    // lanes per column (power of two, <= 64)
@@ -164,9 +174,24 @@ __global__ __launch_bounds__(1024) void retention_kernel(RetentionParams p) {
   float* ks = qs + TC * QS;
   float* vs = ks + TC * QS;               // [TC][V]
   float* os = vs + TC * p.V;              // [TC][V]
-  const int b = blockIdx.x, h = blockIdx.y;
-  const int r0 = p.q_start ? p.q_start[b] : b;
-  const int r1 = p.q_start ? p.q_start[b + 1] : b + 1;
+  int b = blockIdx.x;
+  const int h = blockIdx.y;
+  int r0, r1;
+  if (MODE == 0) {
+    r0 = p.q_start ? p.q_start[b] : b;
+    r1 = p.q_start ? p.q_start[b + 1] : b + 1;
+  } else {
+    // blockIdx.x is a segment entry: its sequence is the last one whose base is not above it
+    int lo = 0, hi = p.num_seqs - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (seg_base(p.q_start, mid, p.SEG) <= (int)blockIdx.x) lo = mid; else hi = mid - 1;
+    }
+    b = lo;
+    const int sg = blockIdx.x - seg_base(p.q_start, b, p.SEG);
+    r0 = p.q_start[b] + sg * p.SEG;
+    r1 = min(r0 + p.SEG, p.q_start[b + 1]);
+  }
   if (r1 <= r0) return;
   const int slot = p.seq_slot[r0];
   if (slot < 0 || slot >= p.num_slots) return;
@@ -174,9 +199,11 @@ __global__ __launch_bounds__(1024) void retention_kernel(RetentionParams p) {
   const int v = tid / DP, part = tid % DP;
   const bool owner = v < p.V;
   const int d0 = part * DREG;
-  float* sp = p.state + (((size_t)slot * p.H + h) * p.V + (owner ? v : 0)) * p.D + d0;
+  float* sp = MODE == 0
+      ? p.state + (((size_t)slot * p.H + h) * p.V + (owner ? v : 0)) * p.D + d0
+      : p.seg_buf + (((size_t)blockIdx.x * p.H + h) * p.V + (owner ? v : 0)) * p.D + d0;
   float S[DREG];
-  const bool fresh = p.positions[r0] == 0;
+  const bool fresh = MODE == 1 || (MODE == 0 && p.positions[r0] == 0);
 #pragma unroll
   for (int i = 0; i < DREG; ++i) S[i] = (!fresh && owner && d0 + i < p.D) ? sp[i] : 0.f;
   const float decay = exp2f(p.log2_decay[h]);
@@ -236,15 +263,20 @@ __global__ __launch_bounds__(1024) void retention_kernel(RetentionParams p) {
         S[i + 1] = fmaf(decay, S[i + 1], k4.y * vv);
         S[i + 2] = fmaf(decay, S[i + 2], k4.z * vv);
         S[i + 3] = fmaf(decay, S[i + 3], k4.w * vv);
-        acc = fmaf(S[i], q4.x, acc);
-        acc = fmaf(S[i + 1], q4.y, acc);
-        acc = fmaf(S[i + 2], q4.z, acc);
-        acc = fmaf(S[i + 3], q4.w, acc);
+        if (MODE != 1) {
+          acc = fmaf(S[i], q4.x, acc);
+          acc = fmaf(S[i + 1], q4.y, acc);
+          acc = fmaf(S[i + 2], q4.z, acc);
+          acc = fmaf(S[i + 3], q4.w, acc);
+        }
       }
-      for (int o = DP >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-      if (owner && part == 0) os[tk * p.V + v] = acc;
+      if (MODE != 1) {
+        for (int o = DP >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+        if (owner && part == 0) os[tk * p.V + v] = acc;
+      }
     }
     __syncthreads();
+    if (MODE == 1) continue;
     // output norm over the head's V entries and the silu gate
     for (int tk = wave; tk < n; tk += nw) {
       float ss = 0.f;
@@ -263,10 +295,36 @@ __global__ __launch_bounds__(1024) void retention_kernel(RetentionParams p) {
     }
     __syncthreads();
   }
-  if (owner) {
+  if (owner && MODE != 3) {
 #pragma unroll
     for (int i = 0; i < DREG; ++i)
       if (d0 + i < p.D) sp[i] = S[i];
+  }
+}
+
+// state before each segment from the segments' own states, per (sequence, head); the state
+// after the last segment goes to the sequence's slot
+__global__ __launch_bounds__(256) void retention_scan_kernel(RetentionParams p) {
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int r0 = p.q_start[b], r1 = p.q_start[b + 1];
+  if (r1 <= r0) return;
+  const int slot = p.seq_slot[r0];
+  if (slot < 0 || slot >= p.num_slots) return;
+  const int n = r1 - r0, nseg = (n + p.SEG - 1) / p.SEG;
+  const bool fresh = p.positions[r0] == 0;
+  const float l2 = p.log2_decay[h];
+  const size_t hs = (size_t)p.V * p.D;
+  float* st = p.state + ((size_t)slot * p.H + h) * hs;
+  float* sb = p.seg_buf + ((size_t)seg_base(p.q_start, b, p.SEG) * p.H + h) * hs;
+  for (int e = threadIdx.x; e < p.V * p.D; e += 256) {
+    float prev = fresh ? 0.f : st[e];
+    for (int sg = 0; sg < nseg; ++sg) {
+      float* cell = sb + (size_t)sg * p.H * hs + e;
+      const float own = *cell;
+      *cell = prev;
+      prev = fmaf(exp2f(l2 * (float)min(p.SEG, n - sg * p.SEG)), prev, own);
+    }
+    st[e] = prev;
   }
 }
 
@@ -615,14 +673,33 @@ void launch_retention(RetentionParams p, bool f32, hipStream_t s) {
     p.TC = RET_TC / 2;
     lds /= 2;
   }
-  const dim3 grid(p.num_seqs, p.H);
-#define AKAP_RET(TY, R) retention_kernel<TY, R><<<grid, nt, lds, s>>>(p)
-  if (f32) {
-    if (dreg == 16) AKAP_RET(float, 16); else if (dreg == 32) AKAP_RET(float, 32); else AKAP_RET(float, 64);
-  } else {
-    if (dreg == 16) AKAP_RET(bf16, 16); else if (dreg == 32) AKAP_RET(bf16, 32); else AKAP_RET(bf16, 64);
+#define AKAP_RET1(TY, R, M) retention_kernel<TY, R, M><<<grid, nt, lds, s>>>(p)
+#define AKAP_RET(M)                                                                   \
+  do {                                                                                \
+    if (f32) {                                                                        \
+      if (dreg == 16) AKAP_RET1(float, 16, M); else if (dreg == 32) AKAP_RET1(float, 32, M); \
+      else AKAP_RET1(float, 64, M);                                                   \
+    } else {                                                                          \
+      if (dreg == 16) AKAP_RET1(bf16, 16, M); else if (dreg == 32) AKAP_RET1(bf16, 32, M);   \
+      else AKAP_RET1(bf16, 64, M);                                                    \
+    }                                                                                 \
+  } while (0)
+  if (p.seg_buf == nullptr) {
+    const dim3 grid(p.num_seqs, p.H);
+    AKAP_RET(0);
+    return;
+  }
+  {
+    const dim3 grid(p.num_segs, p.H);
+    AKAP_RET(1);
+  }
+  retention_scan_kernel<<<dim3(p.num_seqs, p.H), 256, 0, s>>>(p);
+  {
+    const dim3 grid(p.num_segs, p.H);
+    AKAP_RET(3);
   }
 #undef AKAP_RET
+#undef AKAP_RET1
 }
 
 size_t talking_attention_lds(int H, int D) {

@@ -200,6 +200,10 @@ struct RetentionParams {
   const float* log2_decay;   // [H]
   int num_seqs, H, D, V;
   float eps;
+  // segmented form (long prompt chunks, q_start given): states of the segments of SEG rows,
+  // [num_segs, H, V, D] with num_segs = T / SEG + num_seqs; null: the direct form
+  float* seg_buf;
+  int SEG, num_segs;
   int DP, TC;           // set by the launcher
 };
 // 0 when the sizes do not fit a workgroup (V columns x ceil(D / 64) lanes > 1024 threads)

@@ -760,7 +760,7 @@ void head_norm_cache(Tensor proj, Tensor q_out, Tensor k_cache, Tensor v_cache, 
 void retention(Tensor out, Tensor proj, int64_t q_off, int64_t k_off, int64_t v_off, int64_t g_off,
                Tensor state, Tensor seq_slot, Tensor positions, std::optional<Tensor> q_start,
                std::optional<Tensor> cos_sin, Tensor log2_decay, int64_t H, int64_t D, int64_t V,
-               double eps) {
+               double eps, std::optional<Tensor> seg_buf, int64_t seg) {
   CHECK_GPU(out); CHECK_GPU(proj); CHECK_GPU(state); CHECK_GPU(seq_slot); CHECK_GPU(positions);
   CHECK_GPU(log2_decay);
   CHECK_LAST_CONTIG(out); CHECK_LAST_CONTIG(proj); CHECK_CONTIG(state); CHECK_F32(state);
@@ -805,6 +805,15 @@ void retention(Tensor out, Tensor proj, int64_t q_off, int64_t k_off, int64_t v_
   }
   p.log2_decay = log2_decay.data_ptr<float>();
   p.H = H; p.D = D; p.V = V; p.eps = (float)eps; p.DP = 1;
+  p.seg_buf = nullptr; p.SEG = 0; p.num_segs = 0;
+  if (seg_buf.has_value()) {
+    CHECK_GPU(*seg_buf); CHECK_CONTIG(*seg_buf); CHECK_F32(*seg_buf);
+    p.SEG = seg;
+    TORCH_CHECK(q_start.has_value() && seg >= 16, "retention: segments need q_start and >= 16 rows");
+    p.num_segs = T / seg + p.num_seqs;
+    TORCH_CHECK(seg_buf->numel() >= (int64_t)p.num_segs * H * V * D, "retention: seg_buf size");
+    p.seg_buf = seg_buf->data_ptr<float>();
+  }
   const c10::DeviceGuard g(proj.device());
   akap_stream::launch_retention(p, f32, cur_stream());
 }
@@ -1024,7 +1033,8 @@ TORCH_LIBRARY(akap_stream, m) {
         "bool norm_qk, bool norm_v) -> ()");
   m.def("retention(Tensor(a!) out, Tensor proj, int q_off, int k_off, int v_off, int g_off, "
         "Tensor(b!) state, Tensor seq_slot, Tensor positions, Tensor? q_start, Tensor? cos_sin, "
-        "Tensor log2_decay, int H, int D, int V, float eps) -> ()");
+        "Tensor log2_decay, int H, int D, int V, float eps, Tensor(c!)? seg_buf=None, "
+        "int seg=0) -> ()");
   m.def("talking_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, "
         "Tensor block_tables, Tensor seq_lens, Tensor? q_start, Tensor positions, Tensor? talk, "
         "Tensor? gate, float scale, Tensor(b!)? ws_ml, Tensor(c!)? ws_o, int num_parts) -> ()");

@@ -809,6 +809,11 @@ def rotate_half_(x: torch.Tensor, cs: torch.Tensor) -> torch.Tensor:
     return x
 
 
+# steps of at least this many rows run the retention in segments of RETENTION_SEGMENT rows
+RETENTION_SEGMENTED_ROWS = 1024
+RETENTION_SEGMENT = 256
+
+
 def retention(out: torch.Tensor, proj: torch.Tensor, q_off: int, k_off: int, v_off: int,
               g_off: int, state: torch.Tensor, seq_slot: torch.Tensor, positions: torch.Tensor,
               q_start: Optional[torch.Tensor], cos_sin: Optional[torch.Tensor],
@@ -828,9 +833,16 @@ def retention(out: torch.Tensor, proj: torch.Tensor, q_off: int, k_off: int, v_o
     Rotation, decay, state, the output norm and the gate are fp32.  out may be a column slice
     of wider rows."""
     if _native(proj):
+        seg_buf, T = None, proj.shape[0]
+        if q_start is not None and T >= RETENTION_SEGMENTED_ROWS:
+            # long prompt chunks: the segments of a sequence run side by side (each leaves its
+            # own state, a scan turns these into the state before each segment, a second pass
+            # produces the outputs); the buffer is sized from the step's shape alone
+            n = (T // RETENTION_SEGMENT + q_start.numel() - 1) * H * V * D
+            seg_buf = torch.empty(n, dtype=torch.float32, device=proj.device)
         torch.ops.akap_stream.retention(out, proj, q_off, k_off, v_off, g_off, state, seq_slot,
                                         positions, q_start, cos_sin, log2_decay, H, D, V,
-                                        float(eps))
+                                        float(eps), seg_buf, RETENTION_SEGMENT)
         return
     T = proj.shape[0]
     q = proj[:, q_off:q_off + H * D].float().reshape(T, H, D).clone()

@@ -82,7 +82,7 @@ def _retention_case(dtype, H, D, V, rot, dev, steps, g, slots=3):
     N = H * (2 * D + 2 * V) + 5
     state = torch.zeros(slots, H, V, D, device=dev)
     decay = torch.log2(torch.tensor([0.9 + 0.099 * h / max(1, H - 1) for h in range(H)]))
-    cs = sops.rotary_table(512, rot, 10000.0) if rot else None
+    cs = sops.rotary_table(1024, rot, 10000.0) if rot else None
     outs = []
     for step in steps:
         T = sum(n for _, _, n in step)
@@ -113,6 +113,21 @@ def test_retention_kernel(dtype, H, D, V, rot):
     for a, b in zip(res[0][0], res[1][0]):
         close(b, a, dtype, scale=3.0)
     close(res[1][1], res[0][1], "float32")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,D,V,rot", [(3, 64, 32, 16), (2, 128, 128, 64), (2, 24, 40, 8)])
+def test_retention_kernel_in_segments(dtype, H, D, V, rot):
+    """A step long enough for the segmented form: sequences of many segments, one that goes on
+    from its slot's state, a single row and a padding row among them; then single rows that
+    continue from the states the segmented step left."""
+    steps = [[(2, 0, 10)], [(0, 0, 700), (2, 10, 600), (1, 0, 1), (-1, 0, 3), (3, 0, 257)],
+             [(0, 700, 1), (2, 610, 1), (3, 257, 1)]]
+    assert sum(n for _, _, n in steps[1]) >= sops.RETENTION_SEGMENTED_ROWS
+    res = [_retention_case(dtype, H, D, V, rot, dev, steps, gen(9), slots=4) for dev in ("cpu", "cuda")]
+    for a, b in zip(res[0][0], res[1][0]):
+        close(b, a, dtype, scale=10.0)
+    torch.testing.assert_close(res[1][1].cpu(), res[0][1], rtol=2e-4, atol=2e-3)
 
 
 def _attention_case(dtype, H, G, D, Dv, dev, g, parts, talk=True, gate=True, BS=16):
