@@ -239,6 +239,9 @@ void launch_talking_merge(const TalkParams& p, bool f32, hipStream_t s);
 // the rows of the tile map (tile_seq / tile_row: sequence and first chunk row of a tile of
 // tile_rows tokens, a multiple of 32); launch_talking_merge finishes
 bool talk_mfma_supported(int H, int G, int D, int Dv, int BS);
+// matrix-core form for one query per sequence (q_start null): fills the workspace of the
+// num_parts-way split; launch_talking_merge finishes
+void launch_talking_decode_mfma(const TalkParams& p, hipStream_t s);
 void launch_talking_prefill_mfma(const TalkParams& p, const int32_t* tile_seq,
                                  const int32_t* tile_row, int num_tiles, int tile_rows,
                                  hipStream_t s);

@@ -906,6 +906,21 @@ void talking_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache, Ten
   akap_stream::launch_talking_attention(p, is_f32(q, "q"), cur_stream());
 }
 
+void talking_attention_decode_mfma(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
+                                   Tensor block_tables, Tensor seq_lens, Tensor positions,
+                                   std::optional<Tensor> talk, std::optional<Tensor> gate,
+                                   double scale, Tensor ws_ml, Tensor ws_o, int64_t num_parts) {
+  akap_stream::TalkParams p = talk_params(out, q, k_cache, v_cache, block_tables, seq_lens,
+                                          std::nullopt, positions, talk, gate, scale);
+  TORCH_CHECK(q.scalar_type() == at::kBFloat16 &&
+                  akap_stream::talk_mfma_supported(p.H, p.G, p.D, p.Dv, p.BS) && num_parts >= 1,
+              "talking_attention_decode_mfma: bf16 and sizes the matrix-core kernel takes");
+  talk_workspace(p, ws_ml, ws_o, num_parts);
+  const c10::DeviceGuard g(q.device());
+  akap_stream::launch_talking_decode_mfma(p, cur_stream());
+  akap_stream::launch_talking_merge(p, false, cur_stream());
+}
+
 bool talking_mfma_supported(int64_t H, int64_t G, int64_t D, int64_t Dv, int64_t BS) {
   return akap_stream::talk_mfma_supported((int)H, (int)G, (int)D, (int)Dv, (int)BS);
 }
@@ -1044,6 +1059,9 @@ TORCH_LIBRARY(akap_stream, m) {
         "Tensor block_tables, Tensor seq_lens, Tensor q_start, Tensor positions, Tensor tile_seq, "
         "Tensor tile_row, int tile_rows, int first_row, Tensor? talk, Tensor? gate, float scale, "
         "Tensor(b!) ws_ml, Tensor(c!) ws_o) -> ()");
+  m.def("talking_attention_decode_mfma(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, "
+        "Tensor block_tables, Tensor seq_lens, Tensor positions, Tensor? talk, Tensor? gate, "
+        "float scale, Tensor(b!) ws_ml, Tensor(c!) ws_o, int num_parts) -> ()");
   m.def("route_topk(Tensor(a!) ids, Tensor(b!) w, Tensor h, Tensor router, Tensor? bias) -> ()");
   m.def("swiglu_routed(Tensor(a!) out, Tensor gu, Tensor? ids, Tensor? w, int experts) -> ()");
 }
@@ -1067,6 +1085,7 @@ TORCH_LIBRARY_IMPL(akap_stream, CUDA, m) {
   m.impl("retention", &retention);
   m.impl("talking_attention", &talking_attention);
   m.impl("talking_attention_prefill_mfma", &talking_attention_prefill_mfma);
+  m.impl("talking_attention_decode_mfma", &talking_attention_decode_mfma);
   m.impl("route_topk", &route_topk);
   m.impl("swiglu_routed", &swiglu_routed);
   m.impl("embed_scaled", &embed_scaled);

@@ -180,7 +180,183 @@ __global__ __launch_bounds__(256) void talk_prefill_mfma_kernel(TalkParams p, co
   }
 }
 
+// Decode rows (one query per sequence): one workgroup per (row, key partition).  The 32 columns
+// of a tile are the query HEADS of the token; wave w scores all 128 keys of a step for the
+// key heads w, w + 4, ... (only the columns of a key head's own query heads are kept, and since
+// a column belongs to one wave, its running max and sum stay in that wave), the weights of all
+// heads meet in LDS, and every wave accumulates its share of the (value head, 32 entries)
+// column tiles with the heads as rows: each cached key and value is read once per row for all
+// heads.  The partition's unnormalised sums and (max, sum) go to the workspace of the split
+// form; the merge launch combines the partitions, mixes the heads and gates.
+template <int TPW>
+__global__ __launch_bounds__(256) void talk_decode_mfma_kernel(TalkParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int KS = p.D >> 4;
+  bf16x8* qs = (bf16x8*)smem;                      // [KS][64] Q operands (column = head)
+  bf16x8* ps = qs + KS * 64;                       // [2][4 blocks][2][64] weights of a step
+  float* alpha_s = (float*)(ps + 2 * 4 * 2 * 64);  // [2][32]
+
+  const int t = blockIdx.x, part = blockIdx.y;
+  if (p.seq_lens[t] <= 0) return;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int col = lane & 31, hf = lane >> 5;
+  const int rep = p.H / p.G;
+  const int last = (int)p.positions[t];            // the row sees keys 0 .. last
+  const int steps = (last + 128) >> 7;
+  const int per = (steps + p.num_parts - 1) / p.num_parts;
+  const int lo = part * per * 128;
+  const int hi = min(last + 1, lo + per * 128);    // keys [lo, hi)
+  const int32_t* bt = p.block_tables + (size_t)t * p.max_blocks;
+  const float sc2 = p.scale * 1.44269504088896f;
+  const int DVT = p.Dv >> 5, NT = p.G * DVT;
+  const int my_c = col < p.H ? col / rep : -1;     // key head of this column's query head
+  const bool mine = my_c >= 0 && (my_c & 3) == wave;
+
+  for (int e = tid; e < KS * 64; e += 256) {
+    const int c = e >> 6, ln = e & 63;
+    const int qc = ln & 31, qh = ln >> 5;
+    bf16x8 v;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (bf16)0.f;
+    if (qc < p.H)
+      v = *(const bf16x8*)((const bf16*)p.q + ((size_t)t * p.H + qc) * p.D + 16 * c + 8 * qh);
+    qs[e] = v;
+  }
+  {
+    bf16x8 z;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = (bf16)0.f;
+    for (int e = tid; e < 2 * 4 * 2 * 64; e += 256) ps[e] = z;   // columns past H stay zero
+    if (tid < 64) alpha_s[tid] = 0.f;
+  }
+  f32x16 acc[TPW];
+#pragma unroll
+  for (int k = 0; k < TPW; ++k)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[k][i] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  __syncthreads();
+
+  int buf = 0;
+  for (int key0 = lo; key0 < hi; key0 += 128, buf ^= 1) {
+    for (int cc = wave; cc < p.G; cc += 4) {
+      f32x16 s[4];
+#pragma unroll
+      for (int blk = 0; blk < 4; ++blk) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[blk][i] = 0.f;
+        const int kb = key0 + 32 * blk;
+        if (kb < hi) {
+          const int key = min(kb + swap23(col), hi - 1);
+          const int bi = key / p.BS;
+          const bf16* kp = (const bf16*)p.k_cache +
+                           ((size_t)(bt[bi] * p.G + cc) * p.BS + (key - bi * p.BS)) * p.D + 8 * hf;
+          for (int c = 0; c < KS; ++c)
+            s[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(kp + 16 * c),
+                                                             qs[c * 64 + lane], s[blk], 0, 0, 0);
+        }
+      }
+      // the columns of key head cc's query heads: softmax over the step's 128 keys
+      const bool act = my_c == cc;
+      float bmax = -INFINITY;
+#pragma unroll
+      for (int blk = 0; blk < 4; ++blk)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = key0 + 32 * blk + 16 * (i >> 3) + 8 * hf + (i & 7);
+          s[blk][i] = (act && key < hi) ? s[blk][i] * sc2 : -INFINITY;
+          bmax = fmaxf(bmax, s[blk][i]);
+        }
+      bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+      const float mn = fmaxf(m_run, bmax);
+      const float ms = mn == -INFINITY ? 0.f : mn;
+      const float alpha = __builtin_amdgcn_exp2f(m_run - ms);
+      float psum = 0.f;
+#pragma unroll
+      for (int blk = 0; blk < 4; ++blk) {
+        bf16x8 pb[2];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const float e = __builtin_amdgcn_exp2f(s[blk][i] - ms);
+          psum += e;
+          pb[i >> 3][i & 7] = (bf16)e;
+        }
+        if (act) {
+          ps[((buf * 4 + blk) * 2 + 0) * 64 + lane] = pb[0];
+          ps[((buf * 4 + blk) * 2 + 1) * 64 + lane] = pb[1];
+        }
+      }
+      if (act) {
+        m_run = mn;
+        l_run = l_run * alpha + psum;
+        if (hf == 0) alpha_s[buf * 32 + col] = alpha;
+      }
+    }
+    __syncthreads();
+    float ar[16];
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const float4 a4 = *(const float4*)(alpha_s + buf * 32 + 4 * hf + 8 * (i4 & 1) + 16 * (i4 >> 1));
+      ar[4 * i4] = a4.x; ar[4 * i4 + 1] = a4.y; ar[4 * i4 + 2] = a4.z; ar[4 * i4 + 3] = a4.w;
+    }
+#pragma unroll
+    for (int k = 0; k < TPW; ++k) {
+      const int ti = wave + 4 * k;
+      if (ti < NT) {
+        const int cv = ti / DVT, dv0 = (ti - cv * DVT) << 5;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[k][i] *= ar[i];
+        for (int blk = 0; blk < 4; ++blk) {
+#pragma unroll
+          for (int sl = 0; sl < 2; ++sl) {
+            const int kg = key0 + 32 * blk + 16 * sl;
+            if (kg < hi) {
+              const int kk = min(kg + 8 * hf, hi - 1);
+              const int bi = kk / p.BS;
+              const int off = kk - bi * p.BS;
+              const bf16* vp = (const bf16*)p.v_cache +
+                               ((((size_t)(bt[bi] * p.G + cv) * (p.BS >> 3) + (off >> 3)) * p.Dv) +
+                                dv0 + col) * 8;
+              acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                  ps[((buf * 4 + blk) * 2 + sl) * 64 + lane], *(const bf16x8*)vp, acc[k], 0, 0, 0);
+            }
+          }
+        }
+      }
+    }
+  }
+  // (max, sum) of the columns this wave owns, and the sums of its column tiles
+  const size_t cell = (size_t)t * p.num_parts + part;
+  l_run += __shfl_xor(l_run, 32, 64);
+  if (mine && hf == 0) {
+    p.ws_ml[(cell * p.H + col) * 2] = m_run * 0.6931471805599453f;
+    p.ws_ml[(cell * p.H + col) * 2 + 1] = l_run;
+  }
+  const int GV = p.G * p.Dv;
+#pragma unroll
+  for (int k = 0; k < TPW; ++k) {
+    const int ti = wave + 4 * k;
+    if (ti < NT) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int row = (i & 3) + 4 * hf + 8 * ((i >> 2) & 1) + 16 * (i >> 3);
+        if (row < p.H) p.ws_o[(cell * p.H + row) * GV + (ti << 5) + col] = acc[k][i];
+      }
+    }
+  }
+}
+
 }  // namespace
+
+void launch_talking_decode_mfma(const TalkParams& p, hipStream_t s) {
+  if (p.T <= 0) return;
+  const int NT = p.G * (p.Dv / 32);
+  const dim3 grid(p.T, p.num_parts);
+  const size_t lds = (size_t)(p.D / 16) * 64 * 16 + 2 * 4 * 2 * 64 * 16 + 2 * 32 * sizeof(float);
+  if (NT <= 8) talk_decode_mfma_kernel<2><<<grid, 256, lds, s>>>(p);
+  else if (NT <= 16) talk_decode_mfma_kernel<4><<<grid, 256, lds, s>>>(p);
+  else talk_decode_mfma_kernel<8><<<grid, 256, lds, s>>>(p);
+}
 
 bool talk_mfma_supported(int H, int G, int D, int Dv, int BS) {
   return H <= 32 && D % 16 == 0 && D <= 256 && Dv % 32 == 0 && G * (Dv / 32) <= 32 && BS % 16 == 0;

@@ -358,9 +358,9 @@ class SazepelLM:
         parts, ws = 1, None
         if q.is_cuda:
             parts = sops.talking_attention_parts(T, a.kv_heads, self.max_model_len)
-            ws = self._workspace(T, a, parts) if parts > 1 else None
-        sops.talking_attention(out, q, kc, vc, batch.block_tables, batch.seq_lens, None,
-                               batch.positions, talk, gate, a.scale, ws, parts)
+            ws = self._workspace(T, a, parts)
+        sops.talking_attention_decode(out, q, kc, vc, batch.block_tables, batch.seq_lens,
+                                      batch.positions, talk, gate, a.scale, ws, parts)
 
     def _routed(self, lw: SandwichLayerWeights, h2: torch.Tensor, small: bool) -> torch.Tensor:
         """The routed feed-forward of h2 [T, d] as fp32 [T, d]."""

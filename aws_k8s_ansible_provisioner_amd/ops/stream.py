@@ -698,10 +698,10 @@ def head_norm_cache(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tens
 
 def talking_attention_parts(rows: int, kv_heads: int, max_len: int) -> int:
     """Key partitions of a decode row of talking_attention: static in the batch size and the
-    model length (hipGraph-capturable); about four workgroups per CU, a partition never under
-    128 keys."""
+    model length (hipGraph-capturable); one workgroup per (row, partition), about two per CU,
+    a partition never under 128 keys."""
     max_parts = max(1, -(-max_len // 128))
-    return max(1, min(max_parts, 32, -(-1024 // max(1, rows * kv_heads))))
+    return max(1, min(max_parts, 32, -(-512 // max(1, rows))))
 
 
 def talking_attention_workspace(rows: int, H: int, G: int, Dv: int, parts: int, device):
@@ -760,6 +760,29 @@ def talking_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
         if gate is not None:
             o = o * torch.sigmoid(gate[r0:r1].float())
         out[r0:r1] = o.to(out.dtype)
+
+
+def talking_attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
+                             v_cache: torch.Tensor, block_tables: torch.Tensor,
+                             seq_lens: torch.Tensor, positions: torch.Tensor,
+                             talk: Optional[torch.Tensor], gate: Optional[torch.Tensor],
+                             scale: float, workspace=None, num_parts: int = 1) -> None:
+    """talking_attention with one query per sequence (row t is sequence t; seq_lens 0: a
+    padding row, left unwritten).  On the GPU in bf16, at sizes the matrix-core kernel takes and
+    with a workspace (talking_attention_workspace), the heads of a token are the columns of one
+    matrix tile and every cached key and value is read once per row; the keys are cut into
+    num_parts partitions, one workgroup each, merged, mixed and gated by a second launch."""
+    H, D = q.shape[1], q.shape[2]
+    G, BS, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    if (q.is_cuda and q.dtype == torch.bfloat16 and workspace is not None
+            and load_native(required=True)
+            and torch.ops.akap_stream.talking_mfma_supported(H, G, D, Dv, BS)):
+        torch.ops.akap_stream.talking_attention_decode_mfma(
+            out, q, k_cache, v_cache, block_tables, seq_lens, positions, talk, gate, float(scale),
+            workspace[0], workspace[1], int(num_parts))
+        return
+    talking_attention(out, q, k_cache, v_cache, block_tables, seq_lens, None, positions, talk,
+                      gate, scale, workspace, num_parts)
 
 
 def talking_attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,

@@ -245,6 +245,40 @@ def test_talking_attention_matrix_core_kernel(H, G, D, Dv, BS):
         assert (out[:, H * Dv:] == 0).all()
 
 
+@pytest.mark.parametrize("H,G,D,Dv,BS", [(6, 3, 96, 96, 32), (4, 1, 16, 32, 16), (8, 8, 32, 64, 32),
+                                         (16, 4, 128, 128, 32), (2, 2, 48, 160, 16),
+                                         (32, 8, 64, 128, 32)])
+def test_talking_attention_matrix_core_decode_kernel(H, G, D, Dv, BS):
+    """One query per sequence on the matrix cores (heads as columns), several partition counts,
+    sequences of 1 key, of a few and of many steps, a padding row."""
+    g = gen(H * D + 1)
+    lens = [1, 700, 0, 129, 128, 333, 64]
+    NB = sum(-(-n // BS) for n in lens) + 2
+    kc = torch.randn(NB, G, BS, D, generator=g).bfloat16()
+    vc = torch.randn(NB, G, BS // 8, Dv, 8, generator=g).bfloat16()
+    perm = torch.randperm(NB, generator=g).int()
+    bt = torch.zeros(len(lens), max(-(-n // BS) for n in lens), dtype=torch.int32)
+    o = 0
+    for b, n in enumerate(lens):
+        nb = -(-n // BS)
+        bt[b, :nb] = perm[o:o + nb]
+        o += nb
+    T = len(lens)
+    q = (0.5 * torch.randn(T, H, D, generator=g)).bfloat16()
+    sl = torch.tensor(lens, dtype=torch.int32)
+    pos = (sl - 1).clamp(min=0).long()
+    tk = torch.eye(H) + 0.3 * torch.randn(H, H, generator=g)
+    gt = torch.randn(T, H * Dv, generator=g).bfloat16()
+    want = torch.full((T, H * Dv), 3.0, dtype=torch.bfloat16)
+    sops.talking_attention(want, q, kc, vc, bt, sl, None, pos, tk, gt, 0.3)
+    for parts in (1, 3, 8):
+        out = torch.full((T, H * Dv), 3.0, dtype=torch.bfloat16, device="cuda")
+        ws = sops.talking_attention_workspace(T, H, G, Dv, parts, "cuda")
+        sops.talking_attention_decode(out, q.cuda(), kc.cuda(), vc.cuda(), bt.cuda(), sl.cuda(),
+                                      pos.cuda(), tk.cuda(), gt.cuda(), 0.3, ws, parts)
+        close(out, want, "bfloat16")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("E,top,F_,d", [(16, 3, 96, 192), (5, 5, 7, 40), (8, 1, 64, 256), (3, 2, 8, 24)])
 def test_routing_and_gated_activation_kernels(dtype, E, top, F_, d):
