@@ -87,10 +87,27 @@ __global__ __launch_bounds__(256) void talk_prefill_mfma_kernel(TalkParams p, co
       const int bi = key / p.BS;
       const bf16* kp = (const bf16*)p.k_cache +
                        ((size_t)(bt[bi] * p.G + kvh) * p.BS + (key - bi * p.BS)) * p.D + 8 * hf;
-      for (int c = 0; c < KS; ++c) {
-        const bf16x8 kf = *(const bf16x8*)(kp + 16 * c);
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qs[c * 64 + lane], s, 0, 0, 0);
+      // fragment loads go out in batches ahead of their products (a load per product would
+      // make the step a chain of load latencies)
+      for (int c0 = 0; c0 < KS; c0 += 4) {
+        bf16x8 kf[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (c0 + u < KS) kf[u] = *(const bf16x8*)(kp + 16 * (c0 + u));
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (c0 + u < KS)
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[u], qs[(c0 + u) * 64 + lane], s, 0, 0, 0);
       }
+    }
+    // cache rows of the step's eight 16-key operands of the values (requested before the
+    // softmax, used after it)
+    int vrow[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int kk = min(key0 + 16 * j + 8 * hf, kmax);
+      const int bi = kk / p.BS;
+      vrow[j] = bt[bi] * p.G * (p.BS >> 3) + ((kk - bi * p.BS) >> 3);
     }
     // register i of this lane: key kb + 16 (i >> 3) + 8 hf + (i & 7), query column col
     float bmax = -INFINITY;
@@ -136,23 +153,18 @@ __global__ __launch_bounds__(256) void talk_prefill_mfma_kernel(TalkParams p, co
         const int cv = ti / DVT, dv0 = (ti - cv * DVT) << 5;
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[k][i] *= ar[i];
-        for (int w2 = 0; w2 < 4; ++w2) {
+        // operand j: keys key0 + 16 j ..+16 (a group wholly past the range has weights 0)
+        bf16x8 vf[8];
 #pragma unroll
-          for (int sl = 0; sl < 2; ++sl) {
-            const int kg = key0 + 32 * w2 + 16 * sl;   // first key of this 16-key operand
-            if (kg <= kmax) {
-              const int kk = min(kg + 8 * hf, kmax);   // a group wholly past the range: weights 0
-              const int bi = kk / p.BS;
-              const int off = kk - bi * p.BS;
-              const bf16* vp = (const bf16*)p.v_cache +
-                               ((((size_t)(bt[bi] * p.G + cv) * (p.BS >> 3) + (off >> 3)) * p.Dv) +
-                                dv0 + col) * 8;
-              const bf16x8 vf = *(const bf16x8*)vp;
-              acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                  ps[((buf * 4 + w2) * 2 + sl) * 64 + lane], vf, acc[k], 0, 0, 0);
-            }
-          }
-        }
+        for (int j = 0; j < 8; ++j)
+          if (key0 + 16 * j <= kmax)
+            vf[j] = *(const bf16x8*)((const bf16*)p.v_cache +
+                                     (((size_t)vrow[j] + (size_t)cv * (p.BS >> 3)) * p.Dv + dv0 + col) * 8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (key0 + 16 * j <= kmax)
+            acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ps[(buf * 8 + j) * 64 + lane], vf[j],
+                                                             acc[k], 0, 0, 0);
       }
     }
   }
@@ -241,20 +253,33 @@ __global__ __launch_bounds__(256) void talk_decode_mfma_kernel(TalkParams p) {
   for (int key0 = lo; key0 < hi; key0 += 128, buf ^= 1) {
     for (int cc = wave; cc < p.G; cc += 4) {
       f32x16 s[4];
+      const bf16* kp[4];
 #pragma unroll
       for (int blk = 0; blk < 4; ++blk) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[blk][i] = 0.f;
-        const int kb = key0 + 32 * blk;
-        if (kb < hi) {
-          const int key = min(kb + swap23(col), hi - 1);
-          const int bi = key / p.BS;
-          const bf16* kp = (const bf16*)p.k_cache +
-                           ((size_t)(bt[bi] * p.G + cc) * p.BS + (key - bi * p.BS)) * p.D + 8 * hf;
-          for (int c = 0; c < KS; ++c)
-            s[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(kp + 16 * c),
-                                                             qs[c * 64 + lane], s[blk], 0, 0, 0);
-        }
+        const int key = min(key0 + 32 * blk + swap23(col), hi - 1);
+        const int bi = key / p.BS;
+        kp[blk] = (const bf16*)p.k_cache +
+                  ((size_t)(bt[bi] * p.G + cc) * p.BS + (key - bi * p.BS)) * p.D + 8 * hf;
+      }
+      // the fragments of two 16-wide steps of all four key blocks go out together, ahead of
+      // their products
+      for (int c0 = 0; c0 < KS; c0 += 2) {
+        bf16x8 kf[4][2];
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk)
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+            if (key0 + 32 * blk < hi && c0 + u < KS)
+              kf[blk][u] = *(const bf16x8*)(kp[blk] + 16 * (c0 + u));
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk)
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+            if (key0 + 32 * blk < hi && c0 + u < KS)
+              s[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[blk][u], qs[(c0 + u) * 64 + lane],
+                                                               s[blk], 0, 0, 0);
       }
       // the columns of key head cc's query heads: softmax over the step's 128 keys
       const bool act = my_c == cc;
@@ -292,6 +317,13 @@ __global__ __launch_bounds__(256) void talk_decode_mfma_kernel(TalkParams p) {
         if (hf == 0) alpha_s[buf * 32 + col] = alpha;
       }
     }
+    int vrow[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int kk = min(key0 + 16 * j + 8 * hf, hi - 1);
+      const int bi = kk / p.BS;
+      vrow[j] = bt[bi] * p.G * (p.BS >> 3) + ((kk - bi * p.BS) >> 3);
+    }
     __syncthreads();
     float ar[16];
 #pragma unroll
@@ -306,22 +338,17 @@ __global__ __launch_bounds__(256) void talk_decode_mfma_kernel(TalkParams p) {
         const int cv = ti / DVT, dv0 = (ti - cv * DVT) << 5;
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[k][i] *= ar[i];
-        for (int blk = 0; blk < 4; ++blk) {
+        bf16x8 vf[8];
 #pragma unroll
-          for (int sl = 0; sl < 2; ++sl) {
-            const int kg = key0 + 32 * blk + 16 * sl;
-            if (kg < hi) {
-              const int kk = min(kg + 8 * hf, hi - 1);
-              const int bi = kk / p.BS;
-              const int off = kk - bi * p.BS;
-              const bf16* vp = (const bf16*)p.v_cache +
-                               ((((size_t)(bt[bi] * p.G + cv) * (p.BS >> 3) + (off >> 3)) * p.Dv) +
-                                dv0 + col) * 8;
-              acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                  ps[((buf * 4 + blk) * 2 + sl) * 64 + lane], *(const bf16x8*)vp, acc[k], 0, 0, 0);
-            }
-          }
-        }
+        for (int j = 0; j < 8; ++j)
+          if (key0 + 16 * j < hi)
+            vf[j] = *(const bf16x8*)((const bf16*)p.v_cache +
+                                     (((size_t)vrow[j] + (size_t)cv * (p.BS >> 3)) * p.Dv + dv0 + col) * 8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (key0 + 16 * j < hi)
+            acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ps[(buf * 8 + j) * 64 + lane], vf[j],
+                                                             acc[k], 0, 0, 0);
       }
     }
   }
