@@ -24,6 +24,17 @@ __device__ __forceinline__ void stf(T* p, float v) { *p = (T)v; }
 
 __device__ __forceinline__ float sigmoidf(float z) { return 1.0f / (1.0f + __expf(-z)); }
 
+// 4 consecutive elements (16- resp. 8-byte aligned) as floats
+__device__ __forceinline__ void ld4(const float* p, float (&v)[4]) {
+  const float4 a = *(const float4*)p;
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+}
+__device__ __forceinline__ void ld4(const bf16* p, float (&v)[4]) {
+  const akap::bf16x4 a = *(const akap::bf16x4*)p;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] = (float)a[i];
+}
+
 // 8 consecutive elements (32- resp. 16-byte aligned) as floats
 __device__ __forceinline__ void ld8(const float* p, float (&v)[8]) {
   const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
@@ -146,12 +157,16 @@ __global__ __launch_bounds__(256) void head_norm_cache_kernel(HeadNormParams p) 
 }
 
 // ------------------------------------------------------------------ retention
-// One workgroup per (sequence, head).  A thread owns DREG consecutive state rows d of one
-// state column v: the state S[d][v] stays in registers over the sequence's rows of this step.
-// Rows are staged TC at a time: q and k rotated (fp32) into LDS, then the recurrence runs over
-// the TC tokens without a barrier (the DP lanes that share a column add their partial outputs
-// by lane exchange), then the outputs of the TC tokens are normed and gated, a wave per token.
+// One workgroup per (sequence, head).  The state S[d][v] stays in registers over the sequence's
+// rows of this step: a thread owns RET_VR neighbouring state columns v and, of their rows d,
+// DREG / 4 groups of four (group j of lane part `part` covers d = 4 (j DP + part) ..+4, so that
+// the DP lanes of a column read and write consecutive 16-byte pieces of the stored state and
+// of the staged q / k rows).  Rows are staged TC at a time: q and k rotated (fp32) into LDS,
+// then the recurrence runs over the TC tokens without a barrier (every staged k / q value
+// serves RET_VR columns; the DP lanes that share columns add their partial outputs by lane
+// exchange), then the outputs of the TC tokens are normed and gated, a wave per token.
 constexpr int RET_TC = 16;   // tokens staged at a time (8 when the rows of 16 exceed 64 KB)
+constexpr int RET_VR = 4;    // state columns per thread
 
 // Long prompt chunks run in three launches over segments of p.SEG rows, so that a sequence's
 // segments proceed side by side: MODE 1 leaves each segment's own state (started from zeros, no
@@ -164,16 +179,17 @@ __device__ __forceinline__ int seg_base(const int32_t* q_start, int b, int SEG) 
 }
 
 template <typename T, int DREG, int MODE>
-__global__ __launch_bounds__(1024) void retention_kernel(RetentionParams p) {
+__global__ __launch_bounds__(DREG == 16 ? 256 : 512) void retention_kernel(RetentionParams p) {
   extern __shared__ float lds[];
-  const int DP = p.DP;                    // lanes per column (power of two, <= 64)
-  const int DS = DREG + 4;                // padded part stride of the staged q / k rows
-  const int QS = DP * DS;
+  constexpr int NJ = DREG / 4;
+  const int DP = p.DP;                    // lanes per column group (power of two, <= 64)
+  const int DPD = DP * DREG;              // D rounded up: the staged rows end in zeros
+  const int VP = (p.V + 3) & ~3;
   const int TC = p.TC;
-  float* qs = lds;                        // [TC][DP][DS]
-  float* ks = qs + TC * QS;
-  float* vs = ks + TC * QS;               // [TC][V]
-  float* os = vs + TC * p.V;              // [TC][V]
+  float* qs = lds;                        // [TC][DPD]
+  float* ks = qs + TC * DPD;
+  float* vs = ks + TC * DPD;              // [TC][VP]
+  float* os = vs + TC * VP;               // [TC][VP]
   int b = blockIdx.x;
   const int h = blockIdx.y;
   int r0, r1;
@@ -196,24 +212,86 @@ __global__ __launch_bounds__(1024) void retention_kernel(RetentionParams p) {
   const int slot = p.seq_slot[r0];
   if (slot < 0 || slot >= p.num_slots) return;
   const int tid = threadIdx.x, nt = blockDim.x;
-  const int v = tid / DP, part = tid % DP;
-  const bool owner = v < p.V;
-  const int d0 = part * DREG;
-  float* sp = MODE == 0
-      ? p.state + (((size_t)slot * p.H + h) * p.V + (owner ? v : 0)) * p.D + d0
-      : p.seg_buf + (((size_t)blockIdx.x * p.H + h) * p.V + (owner ? v : 0)) * p.D + d0;
-  float S[DREG];
+  const int v0 = (tid / DP) * RET_VR, part = tid % DP;
+  float* sbase = MODE == 0 ? p.state + ((size_t)slot * p.H + h) * p.V * p.D
+                           : p.seg_buf + ((size_t)blockIdx.x * p.H + h) * p.V * p.D;
+  const bool vec = (p.D & 3) == 0;        // 16-byte pieces of the stored state
+  float S[RET_VR][DREG];
   const bool fresh = MODE == 1 || (MODE == 0 && p.positions[r0] == 0);
 #pragma unroll
-  for (int i = 0; i < DREG; ++i) S[i] = (!fresh && owner && d0 + i < p.D) ? sp[i] : 0.f;
+  for (int r = 0; r < RET_VR; ++r) {
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int d = 4 * (j * DP + part);
+      float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (!fresh && v0 + r < p.V) {
+        const float* sp = sbase + (size_t)(v0 + r) * p.D + d;
+        if (vec) {
+          if (d < p.D) t = *(const float4*)sp;
+        } else {
+          if (d < p.D) t.x = sp[0];
+          if (d + 1 < p.D) t.y = sp[1];
+          if (d + 2 < p.D) t.z = sp[2];
+          if (d + 3 < p.D) t.w = sp[3];
+        }
+      }
+      S[r][4 * j] = t.x; S[r][4 * j + 1] = t.y; S[r][4 * j + 2] = t.z; S[r][4 * j + 3] = t.w;
+    }
+  }
   const float decay = exp2f(p.log2_decay[h]);
   const float kscale = 1.0f / sqrtf((float)p.D);
   const int half = p.rot_dims / 2;
-  const int wave = tid >> 6, lane = tid & 63, nw = nt >> 6;
+  // vector staging: every slice starts and every row strides at a multiple of 4 elements
+  const bool vstage = ((p.D | p.V | half | p.proj_stride | p.q_off | p.k_off | p.v_off) & 3) == 0 &&
+                      ((uintptr_t)p.proj & 15) == 0;
+  // lanes per token of the output phase: all TC tokens of a round at once
+  int LPT = 64;
+  while (LPT * TC > nt && LPT > 1) LPT >>= 1;
   for (int c0 = r0; c0 < r1; c0 += TC) {
     const int n = min(TC, r1 - c0);
     // stage: q, k (rotated, k scaled) and v of this head
-    const int DPD = DP * DREG;                // D rounded up to whole parts: the rest is zeros
+    if (vstage) {
+      // four dimensions per item: few rounds of independent vector loads
+      const int Q4 = DPD >> 2;
+      for (int e = tid; e < n * Q4; e += nt) {
+        const int tk = e / Q4, d = (e - tk * Q4) << 2;
+        const T* row = (const T*)p.proj + (size_t)(c0 + tk) * p.proj_stride;
+        const T* q = row + p.q_off + h * p.D;
+        const T* k = row + p.k_off + h * p.D;
+        float q4[4] = {0.f, 0.f, 0.f, 0.f}, k4[4] = {0.f, 0.f, 0.f, 0.f};
+        if (d < p.D) {
+          ld4(q + d, q4);
+          ld4(k + d, k4);
+          if (d < p.rot_dims) {
+            const int64_t pos = p.positions[c0 + tk];
+            const float* cs = p.cos_sin + (size_t)pos * p.rot_dims;
+            const bool low = d < half;
+            const int i = low ? d : d - half, d2 = low ? d + half : d - half;
+            float c4[4], s4[4], q2[4], k2[4];
+            ld4(cs + i, c4);
+            ld4(cs + half + i, s4);
+            ld4(q + d2, q2);
+            ld4(k + d2, k2);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              const float sn = low ? -s4[u] : s4[u];
+              q4[u] = q4[u] * c4[u] + q2[u] * sn;
+              k4[u] = k4[u] * c4[u] + k2[u] * sn;
+            }
+          }
+        }
+        *(float4*)(qs + tk * DPD + d) = make_float4(q4[0], q4[1], q4[2], q4[3]);
+        *(float4*)(ks + tk * DPD + d) =
+            make_float4(k4[0] * kscale, k4[1] * kscale, k4[2] * kscale, k4[3] * kscale);
+      }
+      const int V4 = VP >> 2;
+      for (int e = tid; e < n * V4; e += nt) {
+        const int tk = e / V4, c = (e - tk * V4) << 2;
+        float v4[4];
+        ld4((const T*)p.proj + (size_t)(c0 + tk) * p.proj_stride + p.v_off + h * p.V + c, v4);
+        *(float4*)(vs + tk * VP + c) = make_float4(v4[0], v4[1], v4[2], v4[3]);
+      }
+    } else {
     for (int e = tid; e < n * DPD; e += nt) {
       const int tk = e / DPD, d = e % DPD;
       const T* row = (const T*)p.proj + (size_t)(c0 + tk) * p.proj_stride;
@@ -228,77 +306,103 @@ __global__ __launch_bounds__(1024) void retention_kernel(RetentionParams p) {
         const int64_t pos = p.positions[c0 + tk];
         const float* cs = p.cos_sin + (size_t)pos * p.rot_dims;
         const int i = d < half ? d : d - half;
-        const float c = cs[i], s = cs[half + i];
+        const float c = cs[i], sn = cs[half + i];
         if (d < half) {
           const float q2 = ldf(q + d + half), k2 = ldf(k + d + half);
-          qv = qv * c - q2 * s;
-          kv = kv * c - k2 * s;
+          qv = qv * c - q2 * sn;
+          kv = kv * c - k2 * sn;
         } else {
           const float q1 = ldf(q + d - half), k1 = ldf(k + d - half);
-          qv = qv * c + q1 * s;
-          kv = kv * c + k1 * s;
+          qv = qv * c + q1 * sn;
+          kv = kv * c + k1 * sn;
         }
       }
-      const int o = tk * QS + (d / DREG) * DS + (d % DREG);
-      qs[o] = qv;
-      ks[o] = kv * kscale;
+      qs[e] = qv;
+      ks[e] = kv * kscale;
     }
-    for (int e = tid; e < n * p.V; e += nt) {
-      const int tk = e / p.V, c = e % p.V;
-      vs[tk * p.V + c] =
-          ldf((const T*)p.proj + (size_t)(c0 + tk) * p.proj_stride + p.v_off + h * p.V + c);
+    for (int e = tid; e < n * VP; e += nt) {
+      const int tk = e / VP, c = e % VP;
+      vs[e] = c < p.V ? ldf((const T*)p.proj + (size_t)(c0 + tk) * p.proj_stride + p.v_off +
+                            h * p.V + c)
+                      : 0.f;
+    }
     }
     __syncthreads();
     // the recurrence
     for (int tk = 0; tk < n; ++tk) {
-      const float vv = owner ? vs[tk * p.V + v] : 0.f;
-      const float* kq = ks + tk * QS + part * DS;
-      const float* qq = qs + tk * QS + part * DS;
-      float acc = 0.f;
+      float4 vv = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (v0 < p.V) vv = *(const float4*)(vs + tk * VP + v0);
+      const float vr[RET_VR] = {vv.x, vv.y, vv.z, vv.w};
+      const float* kq = ks + tk * DPD + 4 * part;
+      const float* qq = qs + tk * DPD + 4 * part;
+      float acc[RET_VR] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < DREG; i += 4) {
-        const float4 k4 = *(const float4*)(kq + i);
-        const float4 q4 = *(const float4*)(qq + i);
-        S[i] = fmaf(decay, S[i], k4.x * vv);
-        S[i + 1] = fmaf(decay, S[i + 1], k4.y * vv);
-        S[i + 2] = fmaf(decay, S[i + 2], k4.z * vv);
-        S[i + 3] = fmaf(decay, S[i + 3], k4.w * vv);
-        if (MODE != 1) {
-          acc = fmaf(S[i], q4.x, acc);
-          acc = fmaf(S[i + 1], q4.y, acc);
-          acc = fmaf(S[i + 2], q4.z, acc);
-          acc = fmaf(S[i + 3], q4.w, acc);
+      for (int j = 0; j < NJ; ++j) {
+        const float4 k4 = *(const float4*)(kq + 4 * j * DP);
+        const float4 q4 = *(const float4*)(qq + 4 * j * DP);
+#pragma unroll
+        for (int r = 0; r < RET_VR; ++r) {
+          S[r][4 * j] = fmaf(decay, S[r][4 * j], k4.x * vr[r]);
+          S[r][4 * j + 1] = fmaf(decay, S[r][4 * j + 1], k4.y * vr[r]);
+          S[r][4 * j + 2] = fmaf(decay, S[r][4 * j + 2], k4.z * vr[r]);
+          S[r][4 * j + 3] = fmaf(decay, S[r][4 * j + 3], k4.w * vr[r]);
+          if (MODE != 1) {
+            acc[r] = fmaf(S[r][4 * j], q4.x, acc[r]);
+            acc[r] = fmaf(S[r][4 * j + 1], q4.y, acc[r]);
+            acc[r] = fmaf(S[r][4 * j + 2], q4.z, acc[r]);
+            acc[r] = fmaf(S[r][4 * j + 3], q4.w, acc[r]);
+          }
         }
       }
       if (MODE != 1) {
-        for (int o = DP >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-        if (owner && part == 0) os[tk * p.V + v] = acc;
+        for (int o = DP >> 1; o > 0; o >>= 1) {
+#pragma unroll
+          for (int r = 0; r < RET_VR; ++r) acc[r] += __shfl_xor(acc[r], o, 64);
+        }
+        if (v0 < p.V && part == 0)
+          *(float4*)(os + tk * VP + v0) = make_float4(acc[0], acc[1], acc[2], acc[3]);
       }
     }
     __syncthreads();
     if (MODE == 1) continue;
-    // output norm over the head's V entries and the silu gate
-    for (int tk = wave; tk < n; tk += nw) {
+    // output norm over the head's V entries and the silu gate: LPT lanes per token
+    for (int tk = tid / LPT; tk < n; tk += nt / LPT) {
+      const int ln = tid % LPT;
       float ss = 0.f;
-      for (int c = lane; c < p.V; c += 64) {
-        const float f = os[tk * p.V + c];
+      for (int c = ln; c < p.V; c += LPT) {
+        const float f = os[tk * VP + c];
         ss += f * f;
       }
-      ss = wave_sum(ss);
+      for (int o = LPT >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
       const float inv = 1.0f / sqrtf(ss / (float)p.V + p.eps);
       const T* g = (const T*)p.proj + (size_t)(c0 + tk) * p.proj_stride + p.g_off + h * p.V;
       T* o = (T*)p.out + (size_t)(c0 + tk) * p.out_stride + h * p.V;
-      for (int c = lane; c < p.V; c += 64) {
+      for (int c = ln; c < p.V; c += LPT) {
         const float z = ldf(g + c);
-        stf(o + c, os[tk * p.V + c] * inv * z * sigmoidf(z));
+        stf(o + c, os[tk * VP + c] * inv * z * sigmoidf(z));
       }
     }
     __syncthreads();
   }
-  if (owner && MODE != 3) {
+  if (MODE != 3) {
 #pragma unroll
-    for (int i = 0; i < DREG; ++i)
-      if (d0 + i < p.D) sp[i] = S[i];
+    for (int r = 0; r < RET_VR; ++r) {
+      if (v0 + r >= p.V) continue;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int d = 4 * (j * DP + part);
+        float* sp = sbase + (size_t)(v0 + r) * p.D + d;
+        if (vec) {
+          if (d < p.D)
+            *(float4*)sp = make_float4(S[r][4 * j], S[r][4 * j + 1], S[r][4 * j + 2], S[r][4 * j + 3]);
+        } else {
+          if (d < p.D) sp[0] = S[r][4 * j];
+          if (d + 1 < p.D) sp[1] = S[r][4 * j + 1];
+          if (d + 2 < p.D) sp[2] = S[r][4 * j + 2];
+          if (d + 3 < p.D) sp[3] = S[r][4 * j + 3];
+        }
+      }
+    }
   }
 }
 
@@ -539,13 +643,15 @@ __global__ __launch_bounds__(1024) void talking_merge_kernel(TalkParams p) {
 #pragma unroll
   for (int g = 0; g < HMAX; ++g) acc[g] = 0.f;
   for (int q = 0; q < p.num_parts; ++q) {
+    // every partition wrote its sums (zeros when it had no keys): the loads of a partition go
+    // out together, unconditionally
     const float* o = p.ws_o + ((size_t)t * p.num_parts + q) * p.H * GV + tid;
+    float part[HMAX];
+#pragma unroll
+    for (int g = 0; g < HMAX; ++g) part[g] = g < p.H ? o[(size_t)g * GV] : 0.f;
 #pragma unroll
     for (int g = 0; g < HMAX; ++g)
-      if (g < p.H) {
-        const float w = wgt[q * p.H + g];
-        if (w != 0.f) acc[g] = fmaf(w, o[(size_t)g * GV], acc[g]);
-      }
+      if (g < p.H) acc[g] = fmaf(wgt[q * p.H + g], part[g], acc[g]);
   }
   talk_finish<T, HMAX>(p, t, tid / p.Dv, tid % p.Dv, acc, inv_l);
 }
@@ -650,12 +756,14 @@ void launch_head_norm_cache(const HeadNormParams& p, bool f32, hipStream_t s) {
 }
 
 int retention_dreg(int D, int V) {
-  // state rows per thread: the fewest of 16 / 32 / 64 that keeps the workgroup within 1024
-  // threads (V columns x D / DREG lanes each, the lanes of a column a power of two)
-  for (int dreg : {16, 32, 64}) {
+  // state rows per thread: 16 (64 state registers, workgroups of at most 256 threads), else 32
+  // (128 registers, at most 512 threads); the workgroup has ceil(V / 4) column groups x
+  // D / DREG lanes each, the lanes of a group a power of two
+  for (int dreg : {16, 32}) {
     int dp = 1;
     while (dp * dreg < D) dp <<= 1;
-    if (dp <= 64 && (int64_t)V * dp <= 1024) return dreg;
+    if (dp <= 64 && (int64_t)((V + RET_VR - 1) / RET_VR) * dp <= (dreg == 16 ? 256 : 512))
+      return dreg;
   }
   return 0;
 }
@@ -666,9 +774,10 @@ void launch_retention(RetentionParams p, bool f32, hipStream_t s) {
   int dp = 1;
   while (dp * dreg < p.D) dp <<= 1;
   p.DP = dp;
-  const int nt = ((p.V * dp + 63) / 64) * 64;
+  const int nt = ((((p.V + RET_VR - 1) / RET_VR) * dp + 63) / 64) * 64;
+  const int vp = (p.V + 3) & ~3;
   p.TC = RET_TC;
-  size_t lds = (size_t)p.TC * (2 * dp * (dreg + 4) + 2 * p.V) * sizeof(float);
+  size_t lds = (size_t)p.TC * (2 * dp * dreg + 2 * vp) * sizeof(float);
   if (lds > 65536) {
     p.TC = RET_TC / 2;
     lds /= 2;
@@ -677,11 +786,9 @@ void launch_retention(RetentionParams p, bool f32, hipStream_t s) {
 #define AKAP_RET(M)                                                                   \
   do {                                                                                \
     if (f32) {                                                                        \
-      if (dreg == 16) AKAP_RET1(float, 16, M); else if (dreg == 32) AKAP_RET1(float, 32, M); \
-      else AKAP_RET1(float, 64, M);                                                   \
+      if (dreg == 16) AKAP_RET1(float, 16, M); else AKAP_RET1(float, 32, M);          \
     } else {                                                                          \
-      if (dreg == 16) AKAP_RET1(bf16, 16, M); else if (dreg == 32) AKAP_RET1(bf16, 32, M);   \
-      else AKAP_RET1(bf16, 64, M);                                                    \
+      if (dreg == 16) AKAP_RET1(bf16, 16, M); else AKAP_RET1(bf16, 32, M);            \
     }                                                                                 \
   } while (0)
   if (p.seg_buf == nullptr) {

@@ -206,7 +206,7 @@ struct RetentionParams {
   int SEG, num_segs;
   int DP, TC;           // set by the launcher
 };
-// 0 when the sizes do not fit a workgroup (V columns x ceil(D / 64) lanes > 1024 threads)
+// 0 when the sizes do not fit a workgroup (ceil(V / 4) column groups x D / 32 lanes > 512)
 int retention_dreg(int D, int V);
 void launch_retention(RetentionParams p, bool f32, hipStream_t s);
 

@@ -780,7 +780,7 @@ void retention(Tensor out, Tensor proj, int64_t q_off, int64_t k_off, int64_t v_
   TORCH_CHECK(seq_slot.numel() >= T && positions.numel() >= T && log2_decay.numel() == H,
               "retention: seq_slot / positions / decay sizes");
   TORCH_CHECK(akap_stream::retention_dreg((int)D, (int)V) > 0,
-              "retention: head sizes too large for one workgroup (V * ceil(D / 64) <= 1024)");
+              "retention: head sizes too large for one workgroup (V / 4 * D / 32 <= 512)");
   akap_stream::RetentionParams p;
   p.out = out.data_ptr(); p.out_stride = out.stride(0);
   p.proj = proj.data_ptr(); p.proj_stride = proj.stride(0);

@@ -25,27 +25,30 @@ namespace {
 
 __device__ __forceinline__ int swap23(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1); }
 
-template <int TPW>
+template <int TPW, int NQ>
 __global__ __launch_bounds__(256) void talk_prefill_mfma_kernel(TalkParams p, const int32_t* tile_seq,
                                                                const int32_t* tile_row,
                                                                int tile_rows) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int KS = p.D >> 4;                         // 16-wide steps of the head size
-  bf16x8* qs = (bf16x8*)smem;                      // [KS][64] Q operands
-  bf16x8* ps = qs + KS * 64;                       // [2][4][2][64] weights of a step
-  float* m_loc = (float*)(ps + 2 * 4 * 2 * 64);    // [2][4][32] each wave's maxima
-  float* alpha_s = m_loc + 2 * 4 * 32;             // [2][32] rescale of the step
-  float* l_s = alpha_s + 2 * 32;                   // [4][32] the waves' sums at the end
+  bf16x8* qs = (bf16x8*)smem;                      // [NQ][KS][64] Q operands
+  bf16x8* ps = qs + NQ * KS * 64;                  // [2][NQ][8][64] weights of a step
+  float* m_loc = (float*)(ps + 2 * NQ * 8 * 64);   // [2][4][NQ][32] each wave's maxima
+  float* alpha_s = m_loc + 2 * 4 * NQ * 32;        // [2][NQ][32] rescale of the step
+  float* l_s = alpha_s + 2 * NQ * 32;              // [4][NQ][32] the waves' sums at the end
 
-  const int sub_per = tile_rows >> 5;
-  const int tile = blockIdx.x / sub_per, sub = blockIdx.x - tile * sub_per;
+  constexpr int QT = 32 * NQ;                      // queries of a workgroup
+  const int sub_per = tile_rows / QT;
+  // the map is sorted by rising work: the grid walks it from its end, longest tiles first
+  const int tslot = blockIdx.x / sub_per, sub = blockIdx.x - tslot * sub_per;
+  const int tile = (int)(gridDim.x / sub_per) - 1 - tslot;
   const int g = blockIdx.y;
   const int b = tile_seq[tile];
-  const int r_first = tile_row[tile] + 32 * sub;
+  const int r_first = tile_row[tile] + QT * sub;
   const int chunk = p.q_start[b + 1] - p.q_start[b];
   if (r_first >= chunk) return;
   const int t0 = p.q_start[b] + r_first;
-  const int nrows = min(32, chunk - r_first);
+  const int nrows = min(QT, chunk - r_first);
   const int pos0 = (int)p.positions[t0];
   const int kmax = pos0 + nrows - 1;               // last key any query of the tile sees
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -55,10 +58,10 @@ __global__ __launch_bounds__(256) void talk_prefill_mfma_kernel(TalkParams p, co
   const float sc2 = p.scale * 1.44269504088896f;   // scores -> log2 units
   const int DVT = p.Dv >> 5, NT = p.G * DVT;       // column tiles of 32 value entries
 
-  // Q operands: lane (col = query, hf) of step c holds Q[t0 + col][16 c + 8 hf ..+8]
-  for (int e = tid; e < KS * 64; e += 256) {
-    const int c = e >> 6, ln = e & 63;
-    const int qc = ln & 31, qh = ln >> 5;
+  // Q operands: lane (col = query, hf) of step c holds Q[t0 + 32 q + col][16 c + 8 hf ..+8]
+  for (int e = tid; e < NQ * KS * 64; e += 256) {
+    const int q = e / (KS * 64), c = (e >> 6) % KS, ln = e & 63;
+    const int qc = 32 * q + (ln & 31), qh = ln >> 5;
     bf16x8 v;
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = (bf16)0.f;
@@ -66,22 +69,32 @@ __global__ __launch_bounds__(256) void talk_prefill_mfma_kernel(TalkParams p, co
       v = *(const bf16x8*)((const bf16*)p.q + ((size_t)(t0 + qc) * p.H + g) * p.D + 16 * c + 8 * qh);
     qs[e] = v;
   }
-  f32x16 acc[TPW];
+  f32x16 acc[TPW][NQ];
 #pragma unroll
   for (int k = 0; k < TPW; ++k)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[k][i] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
-  const int qpos = col < nrows ? pos0 + col : -1;  // -1: an unused column sees nothing
+    for (int q = 0; q < NQ; ++q)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[k][q][i] = 0.f;
+  float m_run[NQ], l_run[NQ];
+  int qpos[NQ];
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+    m_run[q] = -INFINITY;
+    l_run[q] = 0.f;
+    qpos[q] = 32 * q + col < nrows ? pos0 + 32 * q + col : -1;   // -1: an unused column
+  }
   __syncthreads();
 
   int buf = 0;
   for (int key0 = 0; key0 <= kmax; key0 += 128, buf ^= 1) {
-    // ---- scores of my 32 keys
+    // ---- scores of my 32 keys against the NQ query tiles: every K fragment is loaded once
     const int kb = key0 + 32 * wave;
-    f32x16 s;
+    f32x16 s[NQ];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+    for (int q = 0; q < NQ; ++q)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[q][i] = 0.f;
     if (kb <= kmax) {
       const int key = min(kb + swap23(col), kmax);  // rows past the range are masked below
       const int bi = key / p.BS;
@@ -96,12 +109,15 @@ __global__ __launch_bounds__(256) void talk_prefill_mfma_kernel(TalkParams p, co
           if (c0 + u < KS) kf[u] = *(const bf16x8*)(kp + 16 * (c0 + u));
 #pragma unroll
         for (int u = 0; u < 4; ++u)
-          if (c0 + u < KS)
-            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[u], qs[(c0 + u) * 64 + lane], s, 0, 0, 0);
+          if (c0 + u < KS) {
+#pragma unroll
+            for (int q = 0; q < NQ; ++q)
+              s[q] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                  kf[u], qs[(q * KS + c0 + u) * 64 + lane], s[q], 0, 0, 0);
+          }
       }
     }
-    // cache rows of the step's eight 16-key operands of the values (requested before the
-    // softmax, used after it)
+    // cache rows of the step's eight 16-key operands of the values
     int vrow[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -110,50 +126,60 @@ __global__ __launch_bounds__(256) void talk_prefill_mfma_kernel(TalkParams p, co
       vrow[j] = bt[bi] * p.G * (p.BS >> 3) + ((kk - bi * p.BS) >> 3);
     }
     // register i of this lane: key kb + 16 (i >> 3) + 8 hf + (i & 7), query column col
-    float bmax = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int key = kb + 16 * (i >> 3) + 8 * hf + (i & 7);
-      s[i] = key <= qpos ? s[i] * sc2 : -INFINITY;
-      bmax = fmaxf(bmax, s[i]);
+    for (int q = 0; q < NQ; ++q) {
+      float bmax = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key = kb + 16 * (i >> 3) + 8 * hf + (i & 7);
+        s[q][i] = key <= qpos[q] ? s[q][i] * sc2 : -INFINITY;
+        bmax = fmaxf(bmax, s[q][i]);
+      }
+      bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+      if (hf == 0) m_loc[((buf * 4 + wave) * NQ + q) * 32 + col] = bmax;
     }
-    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
-    if (hf == 0) m_loc[(buf * 4 + wave) * 32 + col] = bmax;
     __syncthreads();
-    const float* ml = m_loc + buf * 4 * 32 + col;
-    const float mn = fmaxf(fmaxf(m_run, fmaxf(ml[0], ml[32])), fmaxf(ml[64], ml[96]));
-    const float ms = mn == -INFINITY ? 0.f : mn;    // nothing visible yet: every exp below is 0
-    const float alpha = __builtin_amdgcn_exp2f(m_run - ms);
-    m_run = mn;
-    float psum = 0.f;
-    bf16x8 pb[2];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const float e = __builtin_amdgcn_exp2f(s[i] - ms);
-      psum += e;
-      pb[i >> 3][i & 7] = (bf16)e;
+    for (int q = 0; q < NQ; ++q) {
+      const float* ml = m_loc + (buf * 4 * NQ + q) * 32 + col;
+      const float mn = fmaxf(fmaxf(m_run[q], fmaxf(ml[0], ml[NQ * 32])),
+                             fmaxf(ml[2 * NQ * 32], ml[3 * NQ * 32]));
+      const float ms = mn == -INFINITY ? 0.f : mn;  // nothing visible yet: every exp below is 0
+      const float alpha = __builtin_amdgcn_exp2f(m_run[q] - ms);
+      m_run[q] = mn;
+      float psum = 0.f;
+      bf16x8 pb[2];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float e = __builtin_amdgcn_exp2f(s[q][i] - ms);
+        psum += e;
+        pb[i >> 3][i & 7] = (bf16)e;
+      }
+      l_run[q] = l_run[q] * alpha + psum;
+      ps[((buf * NQ + q) * 8 + 2 * wave) * 64 + lane] = pb[0];
+      ps[((buf * NQ + q) * 8 + 2 * wave + 1) * 64 + lane] = pb[1];
+      if (wave == 0 && hf == 0) alpha_s[(buf * NQ + q) * 32 + col] = alpha;
     }
-    l_run = l_run * alpha + psum;
-    ps[((buf * 4 + wave) * 2 + 0) * 64 + lane] = pb[0];
-    ps[((buf * 4 + wave) * 2 + 1) * 64 + lane] = pb[1];
-    if (wave == 0 && hf == 0) alpha_s[buf * 32 + col] = alpha;
     __syncthreads();
     // ---- O += P V for my column tiles; accumulator register i: query row
     //      (i & 3) + 4 hf + 8 ((i >> 2) & 1) + 16 (i >> 3), value entry col of the tile
-    float ar[16];
+    float ar[NQ][16];
 #pragma unroll
-    for (int i4 = 0; i4 < 4; ++i4) {
-      const float4 a4 = *(const float4*)(alpha_s + buf * 32 + 4 * hf + 8 * (i4 & 1) + 16 * (i4 >> 1));
-      ar[4 * i4] = a4.x; ar[4 * i4 + 1] = a4.y; ar[4 * i4 + 2] = a4.z; ar[4 * i4 + 3] = a4.w;
-    }
+    for (int q = 0; q < NQ; ++q)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const float4 a4 = *(const float4*)(alpha_s + (buf * NQ + q) * 32 + 4 * hf + 8 * (i4 & 1) +
+                                           16 * (i4 >> 1));
+        ar[q][4 * i4] = a4.x; ar[q][4 * i4 + 1] = a4.y; ar[q][4 * i4 + 2] = a4.z;
+        ar[q][4 * i4 + 3] = a4.w;
+      }
 #pragma unroll
     for (int k = 0; k < TPW; ++k) {
       const int ti = wave + 4 * k;
       if (ti < NT) {
         const int cv = ti / DVT, dv0 = (ti - cv * DVT) << 5;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[k][i] *= ar[i];
-        // operand j: keys key0 + 16 j ..+16 (a group wholly past the range has weights 0)
+        // operand j: keys key0 + 16 j ..+16 (a group wholly past the range has weights 0);
+        // every value fragment is loaded once for the NQ query tiles
         bf16x8 vf[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j)
@@ -161,32 +187,44 @@ __global__ __launch_bounds__(256) void talk_prefill_mfma_kernel(TalkParams p, co
             vf[j] = *(const bf16x8*)((const bf16*)p.v_cache +
                                      (((size_t)vrow[j] + (size_t)cv * (p.BS >> 3)) * p.Dv + dv0 + col) * 8);
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-          if (key0 + 16 * j <= kmax)
-            acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ps[(buf * 8 + j) * 64 + lane], vf[j],
-                                                             acc[k], 0, 0, 0);
+        for (int q = 0; q < NQ; ++q) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[k][q][i] *= ar[q][i];
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (key0 + 16 * j <= kmax)
+              acc[k][q] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                  ps[((buf * NQ + q) * 8 + j) * 64 + lane], vf[j], acc[k][q], 0, 0, 0);
+        }
       }
     }
   }
   // ---- the head's (max, sum) and its unnormalised sums
-  l_run += __shfl_xor(l_run, 32, 64);
-  if (hf == 0) l_s[wave * 32 + col] = l_run;
-  __syncthreads();
-  if (wave == 0 && hf == 0 && col < nrows) {
-    const size_t cell = ((size_t)(t0 + col) * p.H + g) * 2;
-    p.ws_ml[cell] = m_run * 0.6931471805599453f;
-    p.ws_ml[cell + 1] = l_s[col] + l_s[32 + col] + l_s[64 + col] + l_s[96 + col];
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+    l_run[q] += __shfl_xor(l_run[q], 32, 64);
+    if (hf == 0) l_s[(wave * NQ + q) * 32 + col] = l_run[q];
   }
+  __syncthreads();
   const int GV = p.G * p.Dv;
 #pragma unroll
-  for (int k = 0; k < TPW; ++k) {
-    const int ti = wave + 4 * k;
-    if (ti < NT) {
+  for (int q = 0; q < NQ; ++q) {
+    if (wave == 0 && hf == 0 && 32 * q + col < nrows) {
+      const size_t cell = ((size_t)(t0 + 32 * q + col) * p.H + g) * 2;
+      const float* lq = l_s + q * 32 + col;
+      p.ws_ml[cell] = m_run[q] * 0.6931471805599453f;
+      p.ws_ml[cell + 1] = lq[0] + lq[NQ * 32] + lq[2 * NQ * 32] + lq[3 * NQ * 32];
+    }
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int row = (i & 3) + 4 * hf + 8 * ((i >> 2) & 1) + 16 * (i >> 3);
-        if (row < nrows)
-          p.ws_o[((size_t)(t0 + row) * p.H + g) * GV + (ti << 5) + col] = acc[k][i];
+    for (int k = 0; k < TPW; ++k) {
+      const int ti = wave + 4 * k;
+      if (ti < NT) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int row = 32 * q + (i & 3) + 4 * hf + 8 * ((i >> 2) & 1) + 16 * (i >> 3);
+          if (row < nrows)
+            p.ws_o[((size_t)(t0 + row) * p.H + g) * GV + (ti << 5) + col] = acc[k][q][i];
+        }
       }
     }
   }
@@ -394,12 +432,20 @@ void launch_talking_prefill_mfma(const TalkParams& p, const int32_t* tile_seq,
                                  hipStream_t s) {
   if (num_tiles <= 0) return;
   const int NT = p.G * (p.Dv / 32);
-  const dim3 grid(num_tiles * (tile_rows / 32), p.H);
-  const size_t lds = (size_t)(p.D / 16) * 64 * 16 + 2 * 4 * 2 * 64 * 16 +
-                     (2 * 4 * 32 + 2 * 32 + 4 * 32) * sizeof(float);
-  if (NT <= 8) talk_prefill_mfma_kernel<2><<<grid, 256, lds, s>>>(p, tile_seq, tile_row, tile_rows);
-  else if (NT <= 16) talk_prefill_mfma_kernel<4><<<grid, 256, lds, s>>>(p, tile_seq, tile_row, tile_rows);
-  else talk_prefill_mfma_kernel<8><<<grid, 256, lds, s>>>(p, tile_seq, tile_row, tile_rows);
+  // two query tiles per workgroup (every key and value fragment serves 64 queries) when the
+  // accumulators of the wave's column tiles leave room for it
+  const int nq = (tile_rows % 64 == 0 && NT <= 16) ? 2 : 1;
+  const dim3 grid(num_tiles * (tile_rows / (32 * nq)), p.H);
+  const size_t lds = (size_t)nq * (p.D / 16) * 64 * 16 + (size_t)2 * nq * 8 * 64 * 16 +
+                     (size_t)nq * (2 * 4 * 32 + 2 * 32 + 4 * 32) * sizeof(float);
+#define AKAP_TP(TP, NQ) \
+  talk_prefill_mfma_kernel<TP, NQ><<<grid, 256, lds, s>>>(p, tile_seq, tile_row, tile_rows)
+  if (nq == 2) {
+    if (NT <= 8) AKAP_TP(2, 2); else AKAP_TP(4, 2);
+  } else {
+    if (NT <= 8) AKAP_TP(2, 1); else if (NT <= 16) AKAP_TP(4, 1); else AKAP_TP(8, 1);
+  }
+#undef AKAP_TP
 }
 
 }  // namespace akap_stream
