@@ -301,20 +301,20 @@ __global__ __launch_bounds__(256) void talk_decode_mfma_kernel(TalkParams p) {
         kp[blk] = (const bf16*)p.k_cache +
                   ((size_t)(bt[bi] * p.G + cc) * p.BS + (key - bi * p.BS)) * p.D + 8 * hf;
       }
-      // the fragments of two 16-wide steps of all four key blocks go out together, ahead of
-      // their products
-      for (int c0 = 0; c0 < KS; c0 += 2) {
-        bf16x8 kf[4][2];
+      // the fragments of four 16-wide steps of all four key blocks go out together, ahead of
+      // their products (a decode step is a chain of memory round trips: the fewer the better)
+      for (int c0 = 0; c0 < KS; c0 += 4) {
+        bf16x8 kf[4][4];
 #pragma unroll
         for (int blk = 0; blk < 4; ++blk)
 #pragma unroll
-          for (int u = 0; u < 2; ++u)
+          for (int u = 0; u < 4; ++u)
             if (key0 + 32 * blk < hi && c0 + u < KS)
               kf[blk][u] = *(const bf16x8*)(kp[blk] + 16 * (c0 + u));
 #pragma unroll
         for (int blk = 0; blk < 4; ++blk)
 #pragma unroll
-          for (int u = 0; u < 2; ++u)
+          for (int u = 0; u < 4; ++u)
             if (key0 + 32 * blk < hi && c0 + u < KS)
               s[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[blk][u], qs[(c0 + u) * 64 + lane],
                                                                s[blk], 0, 0, 0);
@@ -369,24 +369,34 @@ __global__ __launch_bounds__(256) void talk_decode_mfma_kernel(TalkParams p) {
       const float4 a4 = *(const float4*)(alpha_s + buf * 32 + 4 * hf + 8 * (i4 & 1) + 16 * (i4 >> 1));
       ar[4 * i4] = a4.x; ar[4 * i4 + 1] = a4.y; ar[4 * i4 + 2] = a4.z; ar[4 * i4 + 3] = a4.w;
     }
+    // the value operands of two column tiles go out together
 #pragma unroll
-    for (int k = 0; k < TPW; ++k) {
-      const int ti = wave + 4 * k;
-      if (ti < NT) {
-        const int cv = ti / DVT, dv0 = (ti - cv * DVT) << 5;
+    for (int k0 = 0; k0 < TPW; k0 += 2) {
+      bf16x8 vf[2][8];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[k][i] *= ar[i];
-        bf16x8 vf[8];
+      for (int u = 0; u < 2; ++u) {
+        const int ti = wave + 4 * (k0 + u);
+        if (ti < NT) {
+          const int cv = ti / DVT, dv0 = (ti - cv * DVT) << 5;
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-          if (key0 + 16 * j < hi)
-            vf[j] = *(const bf16x8*)((const bf16*)p.v_cache +
-                                     (((size_t)vrow[j] + (size_t)cv * (p.BS >> 3)) * p.Dv + dv0 + col) * 8);
+          for (int j = 0; j < 8; ++j)
+            if (key0 + 16 * j < hi)
+              vf[u][j] = *(const bf16x8*)((const bf16*)p.v_cache +
+                                          (((size_t)vrow[j] + (size_t)cv * (p.BS >> 3)) * p.Dv + dv0 + col) * 8);
+        }
+      }
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-          if (key0 + 16 * j < hi)
-            acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ps[(buf * 8 + j) * 64 + lane], vf[j],
-                                                             acc[k], 0, 0, 0);
+      for (int u = 0; u < 2; ++u) {
+        const int ti = wave + 4 * (k0 + u);
+        if (ti < NT) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[k0 + u][i] *= ar[i];
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (key0 + 16 * j < hi)
+              acc[k0 + u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                  ps[(buf * 8 + j) * 64 + lane], vf[u][j], acc[k0 + u], 0, 0, 0);
+        }
       }
     }
   }
