@@ -53,7 +53,7 @@ def test_post_norm_add_norm_kernel(dtype, d):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("H,G,D,Dv", [(6, 3, 96, 96), (4, 1, 20, 36), (8, 8, 128, 64), (3, 3, 7, 5)])
+@pytest.mark.parametrize("H,G,D,Dv", [(6, 2, 80, 96), (4, 1, 20, 36), (8, 8, 128, 64), (3, 3, 7, 5)])
 def test_head_norm_cache_kernel(dtype, H, G, D, Dv):
     g, dt = gen(H * D), DT[dtype]
     T, NB, BS = 9, 4, 16
@@ -101,7 +101,7 @@ def _retention_case(dtype, H, D, V, rot, dev, steps, g, slots=3):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("H,D,V,rot", [(4, 64, 64, 64), (4, 64, 32, 32), (2, 128, 128, 64),
+@pytest.mark.parametrize("H,D,V,rot", [(3, 64, 64, 32), (5, 64, 32, 64), (2, 128, 128, 64),
                                        (3, 24, 40, 8), (2, 80, 96, 0), (1, 256, 256, 128),
                                        (2, 16, 8, 16)])
 def test_retention_kernel(dtype, H, D, V, rot):
@@ -161,7 +161,7 @@ def _attention_case(dtype, H, G, D, Dv, dev, g, parts, talk=True, gate=True, BS=
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("H,G,D,Dv", [(6, 3, 96, 96), (4, 1, 20, 36), (8, 8, 32, 64),
+@pytest.mark.parametrize("H,G,D,Dv", [(6, 2, 80, 96), (4, 1, 20, 36), (8, 8, 32, 64),
                                       (16, 4, 128, 128), (5, 5, 8, 200)])
 def test_talking_attention_kernel(dtype, H, G, D, Dv):
     want = _attention_case(dtype, H, G, D, Dv, "cpu", gen(3), 1)
@@ -207,7 +207,7 @@ def _tile_map(q_start, first_seq, tile_rows):
             torch.tensor(rows, dtype=torch.int32, device="cuda"))
 
 
-@pytest.mark.parametrize("H,G,D,Dv,BS", [(6, 3, 96, 96, 32), (4, 1, 16, 32, 16), (8, 8, 32, 64, 32),
+@pytest.mark.parametrize("H,G,D,Dv,BS", [(6, 2, 80, 96, 32), (4, 1, 16, 32, 16), (8, 8, 32, 64, 32),
                                          (16, 4, 128, 128, 32), (2, 2, 48, 160, 16),
                                          (32, 8, 64, 128, 32)])
 def test_talking_attention_matrix_core_kernel(H, G, D, Dv, BS):
@@ -245,7 +245,7 @@ def test_talking_attention_matrix_core_kernel(H, G, D, Dv, BS):
         assert (out[:, H * Dv:] == 0).all()
 
 
-@pytest.mark.parametrize("H,G,D,Dv,BS", [(6, 3, 96, 96, 32), (4, 1, 16, 32, 16), (8, 8, 32, 64, 32),
+@pytest.mark.parametrize("H,G,D,Dv,BS", [(6, 2, 80, 96, 32), (4, 1, 16, 32, 16), (8, 8, 32, 64, 32),
                                          (16, 4, 128, 128, 32), (2, 2, 48, 160, 16),
                                          (32, 8, 64, 128, 32)])
 def test_talking_attention_matrix_core_decode_kernel(H, G, D, Dv, BS):
@@ -280,7 +280,7 @@ def test_talking_attention_matrix_core_decode_kernel(H, G, D, Dv, BS):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("E,top,F_,d", [(16, 3, 96, 192), (5, 5, 7, 40), (8, 1, 64, 256), (3, 2, 8, 24)])
+@pytest.mark.parametrize("E,top,F_,d", [(12, 3, 80, 160), (5, 5, 7, 40), (8, 1, 64, 256), (3, 2, 8, 24)])
 def test_routing_and_gated_activation_kernels(dtype, E, top, F_, d):
     g, dt = gen(E * d), DT[dtype]
     T = 13
