@@ -50,7 +50,30 @@ __device__ __forceinline__ void ld8(const bf16* p, float (&v)[8]) {
 // ------------------------------------------------------------------ post-norm + residual + norm
 // one workgroup per row; a thread keeps to its own columns in every phase, so the two LDS rows
 // need no barrier beyond those of the block sums
-template <typename TY, typename TO>
+// 8 weights from column c: a vector of d entries (stride 1) or one number (stride 0)
+__device__ __forceinline__ void ldw8(const float* w, int stride, int c, float (&v)[8]) {
+  if (stride) {
+    ld8(w + c, v);
+  } else {
+    const float f = w[0];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = f;
+  }
+}
+__device__ __forceinline__ void st8(float* p, const float (&v)[8]) {
+  *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
+  *(float4*)(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+__device__ __forceinline__ void st8(bf16* p, const float (&v)[8]) {
+  akap::bf16x8 o;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = (bf16)v[i];
+  *(akap::bf16x8*)p = o;
+}
+
+// VEC: 8 columns per thread and turn, 16-byte accesses (d, the row strides and the pointers are
+// multiples of 8 elements resp. 16 bytes)
+template <typename TY, typename TO, bool VEC>
 __global__ __launch_bounds__(256) void post_norm_add_norm_kernel(
     TO* __restrict__ out, int out_stride, float* __restrict__ x, const TY* __restrict__ ya,
     int ya_stride, const TY* __restrict__ yb, int yb_stride, const float* __restrict__ wa, int was,
@@ -66,15 +89,31 @@ __global__ __launch_bounds__(256) void post_norm_add_norm_kernel(
   float* xr = x + (size_t)row * d;
   TO* o = out + (size_t)row * out_stride;
   const float inv_d = 1.0f / (float)d;
+  constexpr int W = VEC ? 8 : 1;
+  const int c0 = threadIdx.x * W, step = 256 * W;
   float ss = 0.f, sb = 0.f;
-  for (int c = threadIdx.x; c < d; c += 256) {
-    const float f = ldf(a + c);
-    ra[c] = f;
-    ss += f * f;
-    if (b) {
-      const float g = ldf(b + c);
-      rb[c] = g;
-      sb += g * g;
+  for (int c = c0; c < d; c += step) {
+    if (VEC) {
+      float f[8];
+      ld8(a + c, f);
+      st8(ra + c, f);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss += f[i] * f[i];
+      if (b) {
+        ld8(b + c, f);
+        st8(rb + c, f);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sb += f[i] * f[i];
+      }
+    } else {
+      const float f = ldf(a + c);
+      ra[c] = f;
+      ss += f * f;
+      if (b) {
+        const float g = ldf(b + c);
+        rb[c] = g;
+        sb += g * g;
+      }
     }
   }
   ss = block_sum(ss, scratch);
@@ -82,24 +121,68 @@ __global__ __launch_bounds__(256) void post_norm_add_norm_kernel(
     sb = block_sum(sb, scratch);
     const float ia = 1.0f / sqrtf(ss * inv_d + eps), ib = 1.0f / sqrtf(sb * inv_d + eps);
     ss = 0.f;
-    for (int c = threadIdx.x; c < d; c += 256) {
-      const float m = 0.5f * (ra[c] * ia * wa[c * was] + rb[c] * ib * wb[c * wbs]);
-      ra[c] = m;
-      ss += m * m;
+    for (int c = c0; c < d; c += step) {
+      if (VEC) {
+        float fa[8], fb[8], ua[8], ub[8];
+        ld8(ra + c, fa);
+        ld8(rb + c, fb);
+        ldw8(wa, was, c, ua);
+        ldw8(wb, wbs, c, ub);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          fa[i] = 0.5f * (fa[i] * ia * ua[i] + fb[i] * ib * ub[i]);
+          ss += fa[i] * fa[i];
+        }
+        st8(ra + c, fa);
+      } else {
+        const float m = 0.5f * (ra[c] * ia * wa[c * was] + rb[c] * ib * wb[c * wbs]);
+        ra[c] = m;
+        ss += m * m;
+      }
     }
     ss = block_sum(ss, scratch);
   }
   const float im = 1.0f / sqrtf(ss * inv_d + eps);
   float sx = 0.f;
-  for (int c = threadIdx.x; c < d; c += 256) {
-    const float f = (fresh ? 0.f : xr[c]) + ra[c] * im * post_w[c * pws];
-    xr[c] = f;
-    ra[c] = f;
-    sx += f * f;
+  for (int c = c0; c < d; c += step) {
+    if (VEC) {
+      float f[8], xv[8], pw[8];
+      ld8(ra + c, f);
+      ldw8(post_w, pws, c, pw);
+      if (fresh) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) xv[i] = 0.f;
+      } else {
+        ld8(xr + c, xv);
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        f[i] = xv[i] + f[i] * im * pw[i];
+        sx += f[i] * f[i];
+      }
+      st8(xr + c, f);
+      st8(ra + c, f);
+    } else {
+      const float f = (fresh ? 0.f : xr[c]) + ra[c] * im * post_w[c * pws];
+      xr[c] = f;
+      ra[c] = f;
+      sx += f * f;
+    }
   }
   sx = block_sum(sx, scratch);
   const float ix = 1.0f / sqrtf(sx * inv_d + eps);
-  for (int c = threadIdx.x; c < d; c += 256) stf(o + c, ra[c] * ix * next_w[c * nws]);
+  for (int c = c0; c < d; c += step) {
+    if (VEC) {
+      float f[8], nw[8];
+      ld8(ra + c, f);
+      ldw8(next_w, nws, c, nw);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) f[i] = f[i] * ix * nw[i];
+      st8(o + c, f);
+    } else {
+      stf(o + c, ra[c] * ix * next_w[c * nws]);
+    }
+  }
 }
 
 // ------------------------------------------------------------------ per-head norms + cache write
@@ -664,15 +747,35 @@ __global__ __launch_bounds__(256) void route_topk_kernel(int32_t* __restrict__ i
                                                          const float* __restrict__ router,
                                                          const float* __restrict__ bias, int d,
                                                          int n, int top) {
-  extern __shared__ float lds[];   // [n] logits
+  extern __shared__ float lds[];   // [n] logits, then the row as fp32 [d]
+  float* hs = lds + ((n + 3) & ~3);
   const int t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const T* hr = h + (size_t)t * h_stride;
+  for (int c = threadIdx.x; c < d; c += 256) hs[c] = ldf(hr + c);
+  __syncthreads();
+  // a logit per wave and turn; 16-byte pieces of the router row and of the staged input
+  const bool vec = (d & 3) == 0;
   for (int e = wave; e < n; e += 4) {
     const float* wr = router + (size_t)e * d;
-    float a = 0.f;
-    for (int c = lane; c < d; c += 64) a = fmaf(ldf(hr + c), wr[c], a);
-    a = wave_sum(a);
+    float a0 = 0.f, a1 = 0.f;
+    if (vec) {
+      int c = lane * 4;
+      for (; c + 256 < d; c += 512) {
+        const float4 w0 = *(const float4*)(wr + c), w1 = *(const float4*)(wr + c + 256);
+        const float4 x0 = *(const float4*)(hs + c), x1 = *(const float4*)(hs + c + 256);
+        a0 = fmaf(x0.x, w0.x, fmaf(x0.y, w0.y, fmaf(x0.z, w0.z, fmaf(x0.w, w0.w, a0))));
+        a1 = fmaf(x1.x, w1.x, fmaf(x1.y, w1.y, fmaf(x1.z, w1.z, fmaf(x1.w, w1.w, a1))));
+      }
+      if (c < d) {
+        const float4 w0 = *(const float4*)(wr + c);
+        const float4 x0 = *(const float4*)(hs + c);
+        a0 = fmaf(x0.x, w0.x, fmaf(x0.y, w0.y, fmaf(x0.z, w0.z, fmaf(x0.w, w0.w, a0))));
+      }
+    } else {
+      for (int c = lane; c < d; c += 64) a0 = fmaf(hs[c], wr[c], a0);
+    }
+    const float a = wave_sum(a0 + a1);
     if (lane == 0) lds[e] = a + (bias ? bias[e] : 0.f);
   }
   __syncthreads();
@@ -738,14 +841,26 @@ void launch_post_norm_add_norm(void* out, bool out_f32, int out_stride, float* x
                                int rows, int d, float eps, bool fresh, hipStream_t s) {
   if (rows <= 0) return;
   const size_t lds = (size_t)2 * d * sizeof(float);
-#define AKAP_PN(TY, TO)                                                                         \
-  post_norm_add_norm_kernel<TY, TO><<<rows, 256, lds, s>>>(                                     \
+  // 16-byte accesses when every row starts at a multiple of 16 bytes
+  auto al = [](const void* p, int bytes) { return p == nullptr || ((uintptr_t)p % bytes) == 0; };
+  const int ye = y_f32 ? 4 : 2, oe = out_f32 ? 4 : 2;
+  const bool vec = d % 8 == 0 && out_stride % 8 == 0 && ya_stride % 8 == 0 && yb_stride % 8 == 0 &&
+                   al(out, 16) && al(x, 16) && al(ya, 16) && al(yb, 16) && al(wa, 16) &&
+                   al(wb, 16) && al(post_w, 16) && al(next_w, 16) && ye > 0 && oe > 0;
+#define AKAP_PN1(TY, TO, V)                                                                      \
+  post_norm_add_norm_kernel<TY, TO, V><<<rows, 256, lds, s>>>(                                   \
       (TO*)out, out_stride, x, (const TY*)ya, ya_stride, (const TY*)yb, yb_stride, wa, was, wb, \
       wbs, post_w, pws, next_w, nws, d, eps, fresh ? 1 : 0)
+#define AKAP_PN(TY, TO)            \
+  do {                             \
+    if (vec) AKAP_PN1(TY, TO, true); \
+    else AKAP_PN1(TY, TO, false);  \
+  } while (0)
   if (y_f32 && out_f32) AKAP_PN(float, float);
   else if (y_f32) AKAP_PN(float, bf16);
   else if (out_f32) AKAP_PN(bf16, float);
   else AKAP_PN(bf16, bf16);
+#undef AKAP_PN1
 #undef AKAP_PN
 }
 
@@ -853,7 +968,7 @@ void launch_route_topk(int32_t* ids, float* w, const void* h, int h_stride, cons
                        const float* bias, int rows, int d, int n, int top, bool f32,
                        hipStream_t s) {
   if (rows <= 0) return;
-  const size_t lds = (size_t)n * sizeof(float);
+  const size_t lds = (size_t)(((n + 3) & ~3) + d) * sizeof(float);
   if (f32)
     route_topk_kernel<float><<<rows, 256, lds, s>>>(ids, w, (const float*)h, h_stride, router, bias,
                                                     d, n, top);

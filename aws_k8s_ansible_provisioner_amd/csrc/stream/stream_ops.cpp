@@ -957,8 +957,9 @@ void route_topk(Tensor ids, Tensor w, Tensor h, Tensor router, std::optional<Ten
   TORCH_CHECK(h.dim() == 2 && router.dim() == 2 && router.size(1) == h.size(1), "route_topk: shapes");
   const int64_t T = h.size(0), n = router.size(0);
   TORCH_CHECK(ids.scalar_type() == at::kInt && ids.dim() == 2 && ids.size(0) == T &&
-                  w.sizes() == ids.sizes() && ids.size(1) >= 1 && ids.size(1) <= n && n <= 8192,
-              "route_topk: ids / w");
+                  w.sizes() == ids.sizes() && ids.size(1) >= 1 && ids.size(1) <= n &&
+                  (n + h.size(1)) * 4 <= 60000,
+              "route_topk: ids / w (and logits + one input row must fit LDS)");
   const float* bp = nullptr;
   if (bias.has_value()) {
     CHECK_GPU(*bias); CHECK_CONTIG(*bias); CHECK_F32(*bias);

@@ -301,23 +301,24 @@ __global__ __launch_bounds__(256) void talk_decode_mfma_kernel(TalkParams p) {
         kp[blk] = (const bf16*)p.k_cache +
                   ((size_t)(bt[bi] * p.G + cc) * p.BS + (key - bi * p.BS)) * p.D + 8 * hf;
       }
-      // the fragments of four 16-wide steps of all four key blocks go out together, ahead of
-      // their products (a decode step is a chain of memory round trips: the fewer the better)
-      for (int c0 = 0; c0 < KS; c0 += 4) {
-        bf16x8 kf[4][4];
+      // one key block at a time, all of its fragments in flight together: the 32 rows of a
+      // block are consumed whole while their cache lines are still in L1 (fragments of several
+      // blocks side by side touch 4 x 32 rows per wave and evict each other)
 #pragma unroll
-        for (int blk = 0; blk < 4; ++blk)
+      for (int blk = 0; blk < 4; ++blk) {
+        if (key0 + 32 * blk < hi) {
+          for (int c0 = 0; c0 < KS; c0 += 8) {
+            bf16x8 kf[8];
 #pragma unroll
-          for (int u = 0; u < 4; ++u)
-            if (key0 + 32 * blk < hi && c0 + u < KS)
-              kf[blk][u] = *(const bf16x8*)(kp[blk] + 16 * (c0 + u));
+            for (int u = 0; u < 8; ++u)
+              if (c0 + u < KS) kf[u] = *(const bf16x8*)(kp[blk] + 16 * (c0 + u));
 #pragma unroll
-        for (int blk = 0; blk < 4; ++blk)
-#pragma unroll
-          for (int u = 0; u < 4; ++u)
-            if (key0 + 32 * blk < hi && c0 + u < KS)
-              s[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[blk][u], qs[(c0 + u) * 64 + lane],
-                                                               s[blk], 0, 0, 0);
+            for (int u = 0; u < 8; ++u)
+              if (c0 + u < KS)
+                s[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[u], qs[(c0 + u) * 64 + lane],
+                                                                 s[blk], 0, 0, 0);
+          }
+        }
       }
       // the columns of key head cc's query heads: softmax over the step's 128 keys
       const bool act = my_c == cc;

@@ -73,7 +73,9 @@ class SazepelLM:
 
     supports_v_tail = False
     gemm_tunable = True
-    gemm_weight_names = ("w_in", "w_o", "w_ao")
+    # the stacked expert weights are GEMM weights of decode-sized batches too (all experts run
+    # as one GEMM pair there)
+    gemm_weight_names = ("w_in", "w_o", "w_ao", "w_up", "w_down")
     fused_gemm_chain = False
     dtypes = (torch.bfloat16, torch.float32)
     # the retention states of a live sequence sit in one of the scheduler's sequence slots: the
