@@ -37,10 +37,8 @@ from .. import ops
 from ..ops import stream as sops
 from ..parallel.state import ParallelState, get_state
 from .config import LatentAttentionSpec, LayeredConfig, LayerSpec
+from .routed import MOE_DENSE_ROWS, routed_sorted
 from .transformer import AttnBatch
-
-# batches up to this many rows take the all-experts GEMM pair of a routed feed-forward
-MOE_DENSE_ROWS = 256
 
 
 @dataclasses.dataclass
@@ -386,30 +384,20 @@ class PuputarLM:
         T, d = h2.shape
         E = rt.experts
         ids, w = sops.moe_route(h2, lw.router, lw.correction, rt.top, rt.groups, rt.keep)
-        out = torch.empty(T, d, dtype=torch.float32, device=h2.device)
         if small:
+            out = torch.empty(T, d, dtype=torch.float32, device=h2.device)
             up = self._linear(h2, lw.w_up)                       # every expert: [T, E F]
             act = torch.empty_like(up)
             sops.relu2_routed(up, ids, w, E, act)
             sops.moe_combine(out, self._linear(act, lw.w_down), None, ids, w, h2, E)
             return out
-        flat = ids.reshape(-1).long()
-        order = torch.argsort(flat, stable=True)                 # sorted pair -> flat (t, k)
-        counts = torch.bincount(flat, minlength=rt.outputs)[:E].tolist()
-        inv = torch.empty(T * rt.top, dtype=torch.int32, device=h2.device)
-        inv[order] = torch.arange(T * rt.top, dtype=torch.int32, device=h2.device)
-        n_real = sum(counts)
-        xs = h2.index_select(0, order[:n_real] // rt.top)
-        ys = torch.empty(max(1, n_real), d, dtype=h2.dtype, device=h2.device)
-        a = 0
-        for e, c in enumerate(counts):
-            if c:
-                u = F.linear(xs[a:a + c], lw.w_up[e * F_:(e + 1) * F_])
-                sops.relu2(u, u)
-                ys[a:a + c] = F.linear(u, lw.w_down[:, e * F_:(e + 1) * F_])
-                a += c
-        sops.moe_combine(out, ys, inv.view(T, rt.top), ids, w, h2, E)
-        return out
+
+        def expert(e: int, rows: torch.Tensor) -> torch.Tensor:
+            u = F.linear(rows, lw.w_up[e * F_:(e + 1) * F_])
+            sops.relu2(u, u)
+            return F.linear(u, lw.w_down[:, e * F_:(e + 1) * F_])
+
+        return routed_sorted(h2, ids, w, E, rt.outputs, expert)
 
     def forward(self, input_ids: torch.Tensor, batch: AttnBatch, k_caches, v_caches
                 ) -> torch.Tensor:

@@ -40,10 +40,8 @@ from .. import ops
 from ..ops import stream as sops
 from ..parallel.state import ParallelState, get_state
 from .config import AttentionSpec, LayeredConfig, LayerSpec, ParallelMixerSpec, RetentionSpec
+from .routed import MOE_DENSE_ROWS, routed_sorted
 from .transformer import AttnBatch
-
-# batches up to this many rows take the all-experts GEMM pair of a routed feed-forward
-MOE_DENSE_ROWS = 256
 
 
 @dataclasses.dataclass
@@ -371,30 +369,21 @@ class SazepelLM:
         T, d = h2.shape
         E = rt.experts
         ids, w = sops.route_topk(h2, lw.router, lw.router_b, rt.top)
-        out = torch.empty(T, d, dtype=torch.float32, device=h2.device)
         if small:
+            out = torch.empty(T, d, dtype=torch.float32, device=h2.device)
             gu = self._linear(h2, lw.w_up)                       # every expert: [T, E 2F]
             act = torch.empty(T, E * F_, dtype=gu.dtype, device=gu.device)
             sops.swiglu_routed(gu, ids, w, E, act)
             sops.moe_combine(out, self._linear(act, lw.w_down), None, ids, w, h2, E)
             return out
-        flat = ids.reshape(-1).long()
-        order = torch.argsort(flat, stable=True)                 # sorted pair -> flat (t, k)
-        counts = torch.bincount(flat, minlength=E).tolist()
-        inv = torch.empty(T * rt.top, dtype=torch.int32, device=h2.device)
-        inv[order] = torch.arange(T * rt.top, dtype=torch.int32, device=h2.device)
-        xs = h2.index_select(0, order // rt.top)
-        ys = torch.empty(T * rt.top, d, dtype=h2.dtype, device=h2.device)
-        a = 0
-        for e, c in enumerate(counts):
-            if c:
-                gu = F.linear(xs[a:a + c], lw.w_up[e * 2 * F_:(e + 1) * 2 * F_])
-                u = torch.empty(c, F_, dtype=gu.dtype, device=gu.device)
-                sops.swiglu(gu, u)
-                ys[a:a + c] = F.linear(u, lw.w_down[:, e * F_:(e + 1) * F_])
-                a += c
-        sops.moe_combine(out, ys, inv.view(T, rt.top), ids, w, h2, E)
-        return out
+
+        def expert(e: int, rows: torch.Tensor) -> torch.Tensor:
+            gu = F.linear(rows, lw.w_up[e * 2 * F_:(e + 1) * 2 * F_])
+            u = torch.empty(rows.shape[0], F_, dtype=gu.dtype, device=gu.device)
+            sops.swiglu(gu, u)
+            return F.linear(u, lw.w_down[:, e * F_:(e + 1) * F_])
+
+        return routed_sorted(h2, ids, w, E, E, expert)
 
     def forward(self, input_ids: torch.Tensor, batch: AttnBatch, k_caches, v_caches
                 ) -> torch.Tensor:
