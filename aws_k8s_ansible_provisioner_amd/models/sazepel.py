@@ -64,6 +64,7 @@ class SandwichLayerWeights:
     w_down: Optional[torch.Tensor] = None   # [d, E F]
     router: Optional[torch.Tensor] = None   # fp32 [E, d]
     router_b: Optional[torch.Tensor] = None
+    w_down_e: Optional[torch.Tensor] = None  # [E, d, F]: w_down per expert, made on first use
 
 
 class SazepelLM:
@@ -243,6 +244,8 @@ class SazepelLM:
                 raise ValueError(f"{name}: checkpoint shape {tuple(src.shape)} does not fit the "
                                  f"config (wanted {tuple(dst.shape)})")
             dst.copy_(src.reshape(dst.shape).to(dst.dtype))
+        for lw in self.layers:
+            lw.w_down_e = None
         self._scale_final()
 
     @property
@@ -253,7 +256,8 @@ class SazepelLM:
         seen = [self.embed, self.embed_norm, self.final_norm, self.lm_head]
         for lw in self.layers:
             seen += [getattr(lw, f.name) for f in dataclasses.fields(lw)
-                     if f.name != "cos_sin" and isinstance(getattr(lw, f.name), torch.Tensor)]
+                     if f.name not in ("cos_sin", "w_down_e")
+                     and isinstance(getattr(lw, f.name), torch.Tensor)]
         return sum(t.numel() * t.element_size() for t in seen)
 
     # ------------------------------------------------------------------ cache and state
@@ -362,8 +366,16 @@ class SazepelLM:
         sops.talking_attention_decode(out, q, kc, vc, batch.block_tables, batch.seq_lens,
                                       batch.positions, talk, gate, a.scale, ws, parts)
 
+    def _grouped_ok(self, h2: torch.Tensor, ff: int) -> bool:
+        """Can the core library's grouped expert GEMMs run this layer (bf16 on the GPU, the
+        library loaded -- a replay engine that returns logits alone runs without it --, both
+        reduction depths multiples of 64)?"""
+        return (h2.is_cuda and self.dtype == torch.bfloat16 and ops.native_loaded()
+                and h2.shape[1] % 64 == 0 and ff % 64 == 0)
+
     def _routed(self, lw: SandwichLayerWeights, h2: torch.Tensor, small: bool) -> torch.Tensor:
-        """The routed feed-forward of h2 [T, d] as fp32 [T, d]."""
+        """The routed feed-forward of h2 [T, d] (fp32, or the activation type from the grouped
+        GEMMs)."""
         ml = lw.spec.mlp
         rt, F_ = ml.router, ml.ff
         T, d = h2.shape
@@ -376,6 +388,14 @@ class SazepelLM:
             sops.swiglu_routed(gu, ids, w, E, act)
             sops.moe_combine(out, self._linear(act, lw.w_down), None, ids, w, h2, E)
             return out
+
+        if self._grouped_ok(h2, F_):
+            # prompt-sized batches on an engine that has the core library: the framework's
+            # grouped expert GEMMs (device-side sort and tile map, SwiGLU in the epilogue, no
+            # host round trip); they take the down-projections per expert, [E, d, F]
+            if lw.w_down_e is None:
+                lw.w_down_e = lw.w_down.view(d, E, F_).permute(1, 0, 2).contiguous()
+            return ops.fused_moe(h2, lw.w_up.view(E, 2 * F_, d), lw.w_down_e, w, ids)
 
         def expert(e: int, rows: torch.Tensor) -> torch.Tensor:
             gu = F.linear(rows, lw.w_up[e * 2 * F_:(e + 1) * 2 * F_])

@@ -25,6 +25,11 @@ _loaded = False
 _load_error: Optional[str] = None
 
 
+def native_loaded() -> bool:
+    """Is the core library loaded in this process (without trying to load it)?"""
+    return _loaded
+
+
 def load_native(required: bool = False) -> bool:
     """Load ``_C.so`` (torch.ops.akap).  Returns True when available."""
     global _loaded, _load_error

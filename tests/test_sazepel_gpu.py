@@ -435,3 +435,25 @@ def test_registry_model_generates_with_sampling():
                                              ignore_eos=True),
                         prompt_ids=[[5, 6, 7], [9] * 70, [1, 2], [3] * 33, [4] * 5])
     assert [len(o.output_ids) for o in outs] == [20] * 5
+
+
+def test_large_batches_take_the_grouped_expert_gemms():
+    """With the core library loaded, prompt-sized batches of a routed layer run the framework's
+    grouped expert GEMMs (no host round trip); same result as the oracle's experts."""
+    from aws_k8s_ansible_provisioner_amd import ops
+    from aws_k8s_ansible_provisioner_amd.models.config import sazepel_config
+    from aws_k8s_ansible_provisioner_amd.models.sazepel import SazepelLM
+
+    ops.load_native(required=True)
+    cfg = oracle.make_config(width=128, vocab=37, layers=[
+        oracle.make_layer(oracle.ret_spec(2, 16, 16), moe=(6, 2, 64))])
+    W = oracle.random_weights(cfg, seed=3)
+    m = SazepelLM(sazepel_config("g", cfg), "cuda", dtype=torch.bfloat16, max_model_len=64)
+    m.load_state_dict(W)
+    h = torch.randn(300, 128, generator=gen(5)).bfloat16()
+    assert m._grouped_ok(h.cuda(), 64)
+    got = m._routed(m.layers[0], h.cuda(), small=False)
+    want = oracle.routed_experts(h.double(), oracle.sub(W, "l0.mlp."), cfg["layers"][0]["mlp"])
+    torch.testing.assert_close(got.double().cpu(), want, rtol=3e-2, atol=3e-2)
+    dense = m._routed(m.layers[0], h.cuda(), small=True)
+    torch.testing.assert_close(dense.double().cpu(), want, rtol=3e-2, atol=3e-2)
