@@ -277,7 +277,7 @@ __global__ __launch_bounds__(256) void talk_decode_mfma_kernel(TalkParams p) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) z[i] = (bf16)0.f;
     for (int e = tid; e < 2 * 4 * 2 * 64; e += 256) ps[e] = z;   // columns past H stay zero
-    if (tid < 64) alpha_s[tid] = 0.f;
+    if (tid < 64) alpha_s[tid] = 1.f;                            // rows past H: never rescaled
   }
   f32x16 acc[TPW];
 #pragma unroll
@@ -323,14 +323,26 @@ __global__ __launch_bounds__(256) void talk_decode_mfma_kernel(TalkParams p) {
       // the columns of key head cc's query heads: softmax over the step's 128 keys
       const bool act = my_c == cc;
       float bmax = -INFINITY;
+      if (key0 + 128 <= hi) {
+        // a whole step: nothing to mask (lanes of other heads' columns compute along; what
+        // they get is never stored)
 #pragma unroll
-      for (int blk = 0; blk < 4; ++blk)
+        for (int blk = 0; blk < 4; ++blk)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int key = key0 + 32 * blk + 16 * (i >> 3) + 8 * hf + (i & 7);
-          s[blk][i] = (act && key < hi) ? s[blk][i] * sc2 : -INFINITY;
-          bmax = fmaxf(bmax, s[blk][i]);
-        }
+          for (int i = 0; i < 16; ++i) {
+            s[blk][i] *= sc2;
+            bmax = fmaxf(bmax, s[blk][i]);
+          }
+      } else {
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int key = key0 + 32 * blk + 16 * (i >> 3) + 8 * hf + (i & 7);
+            s[blk][i] = key < hi ? s[blk][i] * sc2 : -INFINITY;
+            bmax = fmaxf(bmax, s[blk][i]);
+          }
+      }
       bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
       const float mn = fmaxf(m_run, bmax);
       const float ms = mn == -INFINITY ? 0.f : mn;
@@ -370,6 +382,11 @@ __global__ __launch_bounds__(256) void talk_decode_mfma_kernel(TalkParams p) {
       const float4 a4 = *(const float4*)(alpha_s + buf * 32 + 4 * hf + 8 * (i4 & 1) + 16 * (i4 >> 1));
       ar[4 * i4] = a4.x; ar[4 * i4 + 1] = a4.y; ar[4 * i4 + 2] = a4.z; ar[4 * i4 + 3] = a4.w;
     }
+    // the accumulators are rescaled only when some head's maximum moved (wave-uniform)
+    bool moved = false;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) moved |= ar[i] != 1.0f;
+    const bool rescale = __any(moved);
     // the value operands of two column tiles go out together
 #pragma unroll
     for (int k0 = 0; k0 < TPW; k0 += 2) {
@@ -390,8 +407,10 @@ __global__ __launch_bounds__(256) void talk_decode_mfma_kernel(TalkParams p) {
       for (int u = 0; u < 2; ++u) {
         const int ti = wave + 4 * (k0 + u);
         if (ti < NT) {
+          if (rescale) {
 #pragma unroll
-          for (int i = 0; i < 16; ++i) acc[k0 + u][i] *= ar[i];
+            for (int i = 0; i < 16; ++i) acc[k0 + u][i] *= ar[i];
+          }
 #pragma unroll
           for (int j = 0; j < 8; ++j)
             if (key0 + 16 * j < hi)
