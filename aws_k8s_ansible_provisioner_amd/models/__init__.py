@@ -15,6 +15,10 @@ def model_class(cfg: ModelConfig):
         from .sazepel import SazepelLM
 
         return SazepelLM
+    if cfg.arch == "mudepel":
+        from .mudepel import MudepelLM
+
+        return MudepelLM
     from .transformer import DecoderLM
 
     return DecoderLM

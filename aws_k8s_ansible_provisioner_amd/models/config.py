@@ -103,6 +103,12 @@ class RotarySpec:
     dims: int
     base: float
     scaling: Optional[dict] = None
+    # layout "pairs": entries (2i, 2i+1) turn together; "half": entry i with i + dims/2.
+    # scaling with the keys factor / original / fast / slow is the YaRN rule: frequencies whose
+    # index lies under that of `fast` turns in `original` positions are kept, over that of
+    # `slow` turns divided by factor, blended linearly in the index between, and cos and sin
+    # are multiplied by 0.1 ln(factor) + 1
+    layout: str = "pairs"
 
 
 @dataclasses.dataclass
@@ -131,6 +137,13 @@ class AttentionSpec:
     v_norm: bool = False
     talk: bool = False
     gate_per: str = "head"
+    # pool > 0 (with window > 0): beside the last `window` tokens a query sees one mean key and
+    # mean value for every block of `pool` tokens that lies wholly before its window;
+    # unit_sink: a constant 1 in the softmax denominator (a sink of score 0 without a tensor);
+    # bias: the q / k / v / output projections have biases
+    pool: int = 0
+    unit_sink: bool = False
+    bias: bool = False
 
 
 @dataclasses.dataclass
@@ -153,6 +166,45 @@ class RetentionSpec:
     @property
     def state_floats(self) -> int:
         return self.heads * self.dim * self.vdim
+
+
+@dataclasses.dataclass
+class StateSpaceSpec:
+    """A selective state-space mixer (Mamba-2 form): `heads` heads of `vdim` channels, each with
+    an fp32 state S [state, vdim] per live sequence, S_t = exp(-exp(A_h) dt_t) S_(t-1) +
+    dt_t B_t x_t^T and y_t = S_t^T C_t + D_h x_t; B and C (`groups` groups of `state` entries,
+    shared by neighbouring heads) and x pass a causal per-channel convolution of `conv` taps
+    and silu; the output is gated by silu(z) and RMS-normed in `norm_groups` equal parts."""
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    conv: int
+    norm_groups: int = 1
+    # sizing fields shared with AttentionSpec: nothing is cached per token
+    kv_heads: int = 0
+    chunk: int = 0
+    window: int = 0
+
+    @property
+    def dim(self) -> int:
+        return self.vdim
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
+
+    @property
+    def proj_rows(self) -> int:
+        return 2 * self.inner + 2 * self.groups * self.state + self.heads
+
+    @property
+    def state_floats(self) -> int:
+        return self.heads * self.state * self.vdim
 
 
 @dataclasses.dataclass
@@ -221,8 +273,12 @@ class RouterSpec:
     groups: int = 1
     keep: int = 1
     # "corrected": the rule above.  "logits": the `top` largest of (router h + bias) win and
-    # their weights are the softmax over the winners' logits only
+    # their weights are the softmax over the winners' logits only.  "sigmoid": scores are
+    # sigmoid(router h); a group scores the sum of its `group_top` largest scores; the `top`
+    # largest scores of the kept groups win and weigh their experts as they are (no
+    # renormalisation)
     kind: str = "corrected"
+    group_top: int = 1
 
     @property
     def outputs(self) -> int:
@@ -233,15 +289,20 @@ class RouterSpec:
 class MlpSpec:
     kind: str   # "dense": down(act(up h)) | "moe": routed experts of that form
     ff: int
-    act: str = "relu2"              # "relu2" | "xielu" (two learned numbers per layer) | "swiglu"
+    # "relu2" | "xielu" (two learned numbers per layer) | "swiglu" | "geglu" (gated, tanh form
+    # of gelu on the gate)
+    act: str = "relu2"
     bias: bool = False
     router: Optional[RouterSpec] = None
+    shared_ff: int = 0              # > 0: a gated expert of this width that every token uses
 
 
 @dataclasses.dataclass
 class LayerSpec:
-    type: str                       # "attention" | "latent_attention[_2]" | "retention" | "parallel"
-    mixer: object                   # AttentionSpec | LatentAttentionSpec | RetentionSpec | ParallelMixerSpec
+    # "attention" | "latent_attention[_2]" | "retention" | "parallel" | "mamba2"
+    type: str
+    # AttentionSpec | LatentAttentionSpec | RetentionSpec | ParallelMixerSpec | StateSpaceSpec
+    mixer: object
     mlp: Optional[MlpSpec] = None   # None: the layer has no feed-forward
 
 
@@ -258,6 +319,10 @@ class LayeredConfig(ModelConfig):
     residual_mult: float = 1.0
     norm_groups: int = 1            # RMS norms of the stream run in this many equal parts
     logit_scale: float = 1.0        # logits = head x * logit_scale
+    # > 0: that many residual streams with learned read / mix / write weights per sublayer
+    # (hyper-connections) instead of one stream and a plain sum
+    streams: int = 0
+    logit_softcap: float = 0.0      # > 0: logits <- cap tanh(logits / cap)
 
     def layer_runs(self) -> list:
         """Indices into layer_specs in execution order."""
@@ -274,17 +339,22 @@ class LayeredConfig(ModelConfig):
             m = self.layer_specs[i].mixer
             if isinstance(m, LatentAttentionSpec):
                 n += 0 if m.kv_from is not None else m.cache_dim * es
-            elif isinstance(m, RetentionSpec):
+            elif isinstance(m, (RetentionSpec, StateSpaceSpec)):
                 pass
             elif isinstance(m, ParallelMixerSpec):
                 n += m.left.kv_heads * (m.left.dim + m.left.vdim) * es
             else:
-                n += 2 * m.kv_heads * m.dim * es
+                n += m.kv_heads * (m.dim + m.vdim) * es
+                if m.pool > 0:
+                    n += -(-m.kv_heads * (m.dim + m.vdim) * 4 // m.pool)
         return n
 
     def num_params(self) -> int:
         d = self.hidden_size
         n = 2 * self.vocab_size * d + (2 if self.arch == "sazepel" else d)
+        if self.arch == "mudepel":
+            return self.vocab_size * d + d + sum(_mudepel_layer_params(d, max(self.streams, 0), ls)
+                                                 for ls in self.layer_specs)
         for ls in self.layer_specs:
             m = ls.mixer
             if isinstance(m, (RetentionSpec, ParallelMixerSpec)):
@@ -321,6 +391,21 @@ def _sazepel_layer_params(d: int, ls: "LayerSpec") -> int:
     if ls.mlp is not None:
         e = ls.mlp.router.experts if ls.mlp.router else 1
         n += 2 + 3 * d * ls.mlp.ff * e + (e * (d + 1) if ls.mlp.router else 0)
+    return n
+
+
+def _mudepel_layer_params(d: int, streams: int, ls: "LayerSpec") -> int:
+    m = ls.mixer
+    hc = streams * (streams + 2)
+    if isinstance(m, StateSpaceSpec):
+        n = d * m.proj_rows + m.conv_channels * (m.conv + 1) + 3 * m.heads + m.inner + d * m.inner
+    else:
+        n = (d + 1) * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)) + d * (m.heads * m.vdim + 1)
+    n += d + hc
+    ml = ls.mlp
+    if ml is not None:
+        e = ml.router.experts if ml.router else 1
+        n += d + hc + 3 * d * ml.ff * e + 3 * d * ml.shared_ff + (e * d if ml.router else 0)
     return n
 
 
@@ -547,9 +632,141 @@ def puputar_dict(width: int, layers: list, vocab: int = 32000, eps: float = 1e-6
             "vocab": vocab, "width": width}
 
 
+def _mudepel_attention(m: dict) -> AttentionSpec:
+    rot = m.get("rot")
+    rs = None
+    if rot and int(rot.get("dims") or 0) > 0:
+        rs = RotarySpec(int(rot["dims"]), float(rot["base"]), rot.get("scaling") or None,
+                        layout="half")
+        if rs.dims % 2 or rs.dims > int(m["dim"]):
+            raise ValueError("Mudepel: rot.dims must be even and at most dim")
+        if rs.scaling is not None and not all(k in rs.scaling for k in
+                                              ("factor", "original", "fast", "slow")):
+            raise ValueError("Mudepel: rot.scaling needs factor, original, fast and slow")
+    mask = m.get("mask") or {}
+    spec = AttentionSpec(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]),
+                         vdim=int(m["vdim"]), scale=float(m["scale"]), rot=rs,
+                         window=int(mask.get("size") or 0), sink=False, gate=False,
+                         shared_kv=False, pool=int(mask.get("pool") or 0), unit_sink=True,
+                         bias=True)
+    if spec.heads % spec.kv_heads:
+        raise ValueError("Mudepel: heads must be a multiple of kv_heads")
+    if spec.window <= 0:
+        spec.pool = 0
+    return spec
+
+
+def _mudepel_state_space(m: dict) -> StateSpaceSpec:
+    spec = StateSpaceSpec(heads=int(m["heads"]), vdim=int(m["vdim"]), state=int(m["state"]),
+                          groups=int(m["groups"]), conv=int(m["conv"]),
+                          norm_groups=int(m.get("norm_groups") or 1))
+    if spec.heads % spec.groups or spec.inner % spec.norm_groups or spec.conv < 1:
+        raise ValueError("Mudepel: heads must be a multiple of groups, heads x vdim of "
+                         "norm_groups, and conv at least 1")
+    return spec
+
+
+def mudepel_config(name: str, d: dict, max_position: int = 1 << 20) -> LayeredConfig:
+    """A Mudepel config.json: pre-norm layers (norm weights stored around zero) over several
+    residual streams with learned read / mix / write weights, mixers "attention" (biased
+    projections, rotate-half positions with YaRN scaling, a sliding window plus mean-pooled
+    blocks before it, a constant 1 in the softmax denominator) or "mamba2" (selective
+    state-space), feed-forwards "dense" (gelu-gated) or "moe" (sigmoid router over expert
+    groups, silu-gated experts, optional shared expert), an optional loop over a span of
+    layers, tied embeddings and a tanh cap on the logits."""
+    specs = []
+    for ly in d["layers"]:
+        if ly["type"] == "attention":
+            mixer = _mudepel_attention(ly["mixer"])
+        elif ly["type"] == "mamba2":
+            mixer = _mudepel_state_space(ly["mixer"])
+        else:
+            raise ValueError(f"Mudepel: unknown mixer type {ly['type']!r}")
+        ml = ly.get("mlp")
+        mlp = None
+        if ml is not None:
+            if ml.get("kind") == "dense":
+                mlp = MlpSpec("dense", int(ml["ff"]), act="geglu")
+            elif ml.get("kind") == "moe":
+                rt, gr = ml["router"], ml["router"].get("groups") or {}
+                router = RouterSpec(experts=int(rt["experts"]), top=int(rt["top"]),
+                                    groups=int(gr.get("count") or 1), keep=int(gr.get("keep") or 1),
+                                    kind="sigmoid", group_top=2)
+                if router.experts % router.groups or not 1 <= router.keep <= router.groups \
+                        or not 1 <= router.top <= router.keep * (router.experts // router.groups):
+                    raise ValueError(f"Mudepel: bad router {rt}")
+                sh = ml.get("shared")
+                mlp = MlpSpec("moe", int(ml["expert"]["ff"]), act="swiglu", router=router,
+                              shared_ff=int(sh["ff"]) if sh else 0)
+            else:
+                raise ValueError(f"Mudepel: unknown feed-forward kind {ml.get('kind')!r}")
+        specs.append(LayerSpec(ly["type"], mixer, mlp))
+    lp = d.get("loop")
+    loop = None
+    if lp and int(lp.get("times", 1)) != 1 and int(lp["stop"]) > int(lp["start"]):
+        loop = (int(lp["start"]), int(lp["stop"]), int(lp["times"]))
+        if not (0 <= loop[0] < loop[1] <= len(specs)) or loop[2] < 1:
+            raise ValueError(f"Mudepel: bad loop {lp}")
+    att = [ls.mixer for ls in specs if isinstance(ls.mixer, AttentionSpec)]
+    cfg = LayeredConfig(
+        name=name, hf_id=name, arch="mudepel", vocab_size=int(d["vocab"]),
+        hidden_size=int(d["width"]),
+        intermediate_size=max([ls.mlp.ff for ls in specs if ls.mlp is not None] or [0]),
+        num_layers=0, num_heads=max(ls.mixer.heads for ls in specs),
+        num_kv_heads=max([a.kv_heads for a in att] + [1]),
+        head_dim=max([max(a.dim, a.vdim) for a in att] + [ls.mixer.dim for ls in specs]),
+        rms_eps=float(d["norm"]["eps"]), max_position=max_position, bos_id=0, eos_id=-1,
+        tie_embeddings=True, layer_specs=specs, loop=loop, streams=int(d.get("streams") or 0),
+        logit_softcap=float(d.get("logit_softcap") or 0.0))
+    cfg.num_layers = len(cfg.layer_runs())
+    return cfg
+
+
+def mudepel_dict(width: int, layers: list, vocab: int = 32000, eps: float = 1e-6,
+                 streams: int = 2, logit_softcap: float = 30.0, loop: Optional[tuple] = None
+                 ) -> dict:
+    """A Mudepel config.json dictionary from short layer dicts (random-init benchmarks and
+    tests).  A layer gives either `att` = (heads, kv_heads, dim, vdim) with optional window,
+    pool, rot_dims, base, yarn (a scaling dict), scale, or `ssm` = (heads, vdim, state, groups)
+    with optional conv, norm_groups; and `ff` (dense), or experts / expert_ff / top / groups /
+    keep / shared_ff (routed), or neither."""
+    out = []
+    for ly in layers:
+        if "att" in ly:
+            h, g, dd, vv = ly["att"]
+            m = {"heads": h, "kv_heads": g, "dim": dd, "vdim": vv,
+                 "scale": float(ly.get("scale", dd ** -0.5)),
+                 "rot": {"base": float(ly.get("base", 10000.0)),
+                         "dims": int(ly.get("rot_dims", dd)), "scaling": ly.get("yarn")}}
+            if ly.get("window"):
+                m["mask"] = {"size": int(ly["window"]), "pool": int(ly.get("pool") or 0)}
+            kind = "attention"
+        else:
+            h, vv, n, g = ly["ssm"]
+            m = {"heads": h, "vdim": vv, "state": n, "groups": g, "conv": int(ly.get("conv", 4)),
+                 "norm_groups": int(ly.get("norm_groups", 1))}
+            kind = "mamba2"
+        if ly.get("experts"):
+            mlp = {"kind": "moe", "expert": {"ff": ly["expert_ff"]},
+                   "router": {"experts": ly["experts"], "top": ly["top"],
+                              "groups": {"count": ly.get("groups", 1), "keep": ly.get("keep", 1)}}}
+            if ly.get("shared_ff"):
+                mlp["shared"] = {"ff": ly["shared_ff"]}
+        elif ly.get("ff"):
+            mlp = {"kind": "dense", "ff": ly["ff"]}
+        else:
+            mlp = None
+        out.append({"type": kind, "mixer": m, "mlp": mlp})
+    d = {"architecture": "Mudepel", "layers": out, "logit_softcap": logit_softcap,
+         "norm": {"eps": eps}, "streams": streams, "vocab": vocab, "width": width}
+    if loop:
+        d["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return d
+
+
 # config.json readers of designs that do not use the HF key set, by their "architecture" value
 _NATIVE_READERS = {"Bidetar": bidetar_config, "Puputar": puputar_config,
-                   "Sazepel": sazepel_config}
+                   "Sazepel": sazepel_config, "Mudepel": mudepel_config}
 
 _REGISTRY: dict[str, ModelConfig] = {}
 
@@ -767,6 +984,48 @@ SAZEPEL_W4096 = register(_sazepel_stack(
 TINY_SAZEPEL = register(_sazepel_stack(
     "tiny-sazepel", width=128, n=4, att=(4, 2, 32, 16), ret=(2, 16, 32), experts=6, expert_ff=64,
     top=2, vocab=512, rot_dims=8, logit_scale=1.5))
+
+
+def _mudepel_stack(name: str, width: int, n: int, att: tuple, ssm: tuple, ff: int, experts: int,
+                   expert_ff: int, top: int, window: int, pool: int, vocab: int = 32000,
+                   streams: int = 4, groups: int = 1, keep: int = 1, norm_groups: int = 1,
+                   loop: Optional[tuple] = None, rot_dims: Optional[int] = None,
+                   yarn: Optional[dict] = None) -> LayeredConfig:
+    """n layers alternating state-space (dense gelu-gated feed-forward) and windowed attention
+    with pooled blocks (routed feed-forward with a shared expert)."""
+    layers = []
+    for i in range(n):
+        if i % 2 == 0:
+            layers.append(dict(ssm=ssm, norm_groups=norm_groups, ff=ff))
+        else:
+            ly = dict(att=att, window=window, pool=pool, base=500000.0, yarn=yarn,
+                      experts=experts, expert_ff=expert_ff, top=top, groups=groups, keep=keep,
+                      shared_ff=expert_ff)
+            if rot_dims is not None:
+                ly["rot_dims"] = rot_dims
+            layers.append(ly)
+    cfg = mudepel_config(name, mudepel_dict(width, layers, vocab=vocab, streams=streams,
+                                            loop=loop))
+    cfg.hf_id = "test/" + name
+    return cfg
+
+
+# Mudepel at layer sizes of real models (random weights; bench.py --compare-design mudepel):
+# state-space layers of width / 32 heads x 64 channels with 128-entry states, attention layers
+# of 16 / 4 heads of 128 over a 1024-token window and 64-token pooled blocks, 8 experts of
+# which 2 per token beside a shared one
+_YARN = {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+MUDEPEL_W2048 = register(_mudepel_stack(
+    "mudepel-w2048", width=2048, n=16, att=(16, 4, 128, 128), ssm=(64, 64, 128, 1), ff=5632,
+    experts=8, expert_ff=1408, top=2, window=1024, pool=64, yarn=_YARN))
+MUDEPEL_W4096 = register(_mudepel_stack(
+    "mudepel-w4096", width=4096, n=8, att=(32, 8, 128, 128), ssm=(128, 64, 128, 8), ff=11008,
+    experts=8, expert_ff=3584, top=2, window=1024, pool=64, norm_groups=8, yarn=_YARN))
+TINY_MUDEPEL = register(_mudepel_stack(
+    "tiny-mudepel", width=128, n=4, att=(4, 2, 32, 16), ssm=(4, 16, 16, 2), ff=192, experts=6,
+    expert_ff=64, top=2, window=24, pool=8, vocab=512, streams=3, groups=3, keep=2,
+    norm_groups=2, loop=(1, 3, 2), rot_dims=16,
+    yarn={"factor": 2.0, "original": 64, "fast": 8.0, "slow": 1.0}))
 
 
 def get_config(name: str) -> ModelConfig:

@@ -943,3 +943,335 @@ def swiglu_routed(gu: torch.Tensor, ids: torch.Tensor, w: torch.Tensor, experts:
     g3 = gu.float().view(T, experts, 2, F_)
     act = torch.nn.functional.silu(g3[:, :, 0]) * g3[:, :, 1] * full[:, :, None]
     out.copy_(act.view(T, experts * F_).to(out.dtype))
+
+
+# ----------------------------------------------------------------------------- residual streams
+def hyper_step(xs: torch.Tensor, ya: Optional[torch.Tensor], yb: Optional[torch.Tensor],
+               bias: Optional[torch.Tensor], mix: Optional[torch.Tensor],
+               w_out: Optional[torch.Tensor], w_in: torch.Tensor, norm_w: torch.Tensor,
+               eps: float, out: torch.Tensor, fresh: Optional[torch.Tensor] = None) -> None:
+    """One step of a model with S residual streams xs [T, S, d] (fp32, updated in place): the
+    write of a sublayer's output fused with the read and norm that feed the next sublayer.
+    With y = ya + yb + bias (each may be None; [T, d] in the activation type or fp32, bias [d]):
+    every stream at once from the old ones, xs[:, r] <- sum_s mix[s, r] xs[:, s] + w_out[r] y;
+    then u = sum_s w_in[s] xs[:, s] and out = u / sqrt(mean(u^2) + eps) * norm_w.  fresh [T, d]
+    (fp32): instead of an update every stream is set to it (the start of the stack).  mix
+    [S, S] (indexed [from, to]), w_out, w_in [S] and norm_w [d] are fp32; S = 1 with ones is a
+    plain residual sum.  All arithmetic is fp32; out is rounded once."""
+    if _native(xs):
+        torch.ops.akap_stream.hyper_step(out, xs, ya, yb, bias, mix, w_out, w_in, norm_w,
+                                         float(eps), fresh)
+        return
+    if fresh is not None:
+        xs.copy_(fresh.float()[:, None, :].expand_as(xs))
+    else:
+        y = torch.zeros(xs.shape[0], xs.shape[2], dtype=torch.float32)
+        for t in (ya, yb, bias):
+            if t is not None:
+                y = y + t.float()
+        xs.copy_(torch.einsum("sr,tsd->trd", mix.float(), xs) + w_out.float()[None, :, None]
+                 * y[:, None, :])
+    u = torch.einsum("s,tsd->td", w_in.float(), xs)
+    out.copy_((_rms(u, eps) * norm_w.float()).to(out.dtype))
+
+
+def softcap_(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """logits <- cap tanh(logits / cap) in place (fp32 arithmetic)."""
+    if _native(logits):
+        torch.ops.akap_stream.softcap_(logits, float(cap))
+        return logits
+    logits.copy_((cap * torch.tanh(logits.float() / cap)).to(logits.dtype))
+    return logits
+
+
+# ----------------------------------------------------------------------------- windowed attention with pooled blocks
+def rotary_table_yarn(max_pos: int, dims: int, base: float, scaling: Optional[dict],
+                      device=None) -> torch.Tensor:
+    """fp32 [max_pos, dims] = [cos | sin] of the angle p f_i, f_i = base^(-2i/dims), i <
+    dims / 2, under the YaRN rule of scaling = {factor, original, fast, slow}: with
+    at(t) = dims ln(original / (2 pi t)) / (2 ln base), lo = max(floor(at(fast)), 0),
+    hi = min(ceil(at(slow)), dims - 1) and r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)
+    the frequency is f_i / factor r_i + f_i (1 - r_i), and cos and sin carry the factor
+    0.1 ln(factor) + 1.  Angles are formed in fp64 and rounded once."""
+    import math
+
+    half = dims // 2
+    i = torch.arange(half, dtype=torch.float64)
+    f = torch.tensor(float(base), dtype=torch.float64) ** (-2.0 * i / dims)
+    m = 1.0
+    if scaling:
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+
+        def at(turns: float) -> float:
+            return dims * math.log(orig / (2 * math.pi * turns)) / (2 * math.log(base))
+
+        lo = max(math.floor(at(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(at(float(scaling["slow"]))), dims - 1)
+        r = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        f = f / factor * r + f * (1.0 - r)
+        m = 0.1 * math.log(factor) + 1.0
+    a = torch.arange(max_pos, dtype=torch.float64)[:, None] * f[None, :]
+    t = torch.cat([torch.cos(a) * m, torch.sin(a) * m], dim=1).to(torch.float32)
+    return t.to(device) if device is not None else t
+
+
+def pool_slots(block_size: int, pool: int) -> int:
+    """Pooled entries a cache page holds: a block of `pool` tokens is stored with the page of
+    its first token, at index (first token's offset in the page) // pool."""
+    return -(-block_size // pool) if pool > 0 else 0
+
+
+def bias_rope_cache(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor,
+                    v_cache: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor,
+                    cos_sin: Optional[torch.Tensor], bias: Optional[torch.Tensor], H: int, G: int,
+                    D: int, Dv: int, q_off: int, k_off: int, v_off: int) -> None:
+    """Per token t of the fused projection proj [T, N]: q = proj[t, q_off : q_off + H D],
+    k = proj[t, k_off : k_off + G D], v = proj[t, v_off : v_off + G Dv], each plus its slice of
+    bias (fp32 [N], laid out like proj's columns; None: no biases); q and k are rotated per head
+    on their first cos_sin.shape[1] dimensions in the rotate-half layout (entry i with
+    i + dims/2) by the table row of positions[t] (fp32).  q goes to q_out [T, H, D]; k to
+    k_cache [NB, G, BS, D] and v to v_cache [NB, G, BS, Dv] (token-major) at slots[t]; slot -1
+    writes nothing."""
+    if _native(proj):
+        torch.ops.akap_stream.bias_rope_cache(proj, q_out, k_cache, v_cache, positions, slots,
+                                              cos_sin, bias, H, G, D, Dv, q_off, k_off, v_off)
+        return
+    T = proj.shape[0]
+    b = bias.float() if bias is not None else torch.zeros(proj.shape[1])
+    q = (proj[:, q_off:q_off + H * D].float() + b[q_off:q_off + H * D]).view(T, H, D).clone()
+    k = (proj[:, k_off:k_off + G * D].float() + b[k_off:k_off + G * D]).view(T, G, D).clone()
+    v = (proj[:, v_off:v_off + G * Dv].float() + b[v_off:v_off + G * Dv]).view(T, G, Dv)
+    if cos_sin is not None:
+        cs = cos_sin[positions.long()]
+        rotate_half_(q, cs)
+        rotate_half_(k, cs)
+    q_out.copy_(q.to(q_out.dtype))
+    BS = k_cache.shape[2]
+    ok = slots >= 0
+    sl = slots[ok].long()
+    k_cache[sl // BS, :, sl % BS] = k[ok].to(k_cache.dtype)
+    v_cache[sl // BS, :, sl % BS] = v[ok].to(v_cache.dtype)
+
+
+def _row_sequences(T: int, q_start: Optional[torch.Tensor]):
+    """(first row, end row) per sequence of a step: from q_start, or one row each."""
+    if q_start is None:
+        return [(t, t + 1) for t in range(T)]
+    qs = q_start.tolist()
+    return [(qs[b], qs[b + 1]) for b in range(len(qs) - 1)]
+
+
+def pool_cache_blocks(k_cache: torch.Tensor, v_cache: torch.Tensor, k_pool: torch.Tensor,
+                      v_pool: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor,
+                      block_tables: torch.Tensor, q_start: Optional[torch.Tensor],
+                      pool: int) -> None:
+    """For every token row whose position p ends a block of `pool` positions ((p + 1) % pool ==
+    0, slot >= 0): the mean (fp32 sum) of the block's `pool` cached keys, as the cache holds
+    them, goes to k_pool [NB, G, pool_slots, D] (fp32) and the mean of its values to v_pool, at
+    the page of the block's first token, index (its offset in the page) // pool.  Runs after the
+    step's cache write.  The rows of sequence b are [q_start[b], q_start[b + 1]) (None: row t is
+    sequence t); its pages are block_tables[b]."""
+    if _native(k_cache):
+        torch.ops.akap_stream.pool_cache_blocks(k_cache, v_cache, k_pool, v_pool, positions, slots,
+                                                block_tables, q_start, int(pool))
+        return
+    BS = k_cache.shape[2]
+    for b, (r0, r1) in enumerate(_row_sequences(positions.shape[0], q_start)):
+        for t in range(r0, r1):
+            p = int(positions[t])
+            if int(slots[t]) < 0 or (p + 1) % pool:
+                continue
+            first = p + 1 - pool
+            pos = torch.arange(first, p + 1)
+            pages = block_tables[b][pos // BS].long()
+            kk = k_cache[pages, :, pos % BS].float().mean(dim=0)
+            vv = v_cache[pages, :, pos % BS].float().mean(dim=0)
+            page, idx = int(block_tables[b][first // BS]), (first % BS) // pool
+            k_pool[page, :, idx] = kk
+            v_pool[page, :, idx] = vv
+
+
+def pooled_window_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
+                            v_cache: torch.Tensor, k_pool: Optional[torch.Tensor],
+                            v_pool: Optional[torch.Tensor], block_tables: torch.Tensor,
+                            q_start: Optional[torch.Tensor], positions: torch.Tensor,
+                            slots: torch.Tensor, scale: float, window: int, pool: int,
+                            unit_sink: bool) -> None:
+    """Paged attention of the token rows of a step.  The query at position i of sequence b
+    (rows by q_start as in pool_cache_blocks) sees the cached tokens j <= i with i - j < window
+    (window 0: all) and, with pool > 0, the pooled entry of every block c with
+    c pool + pool - 1 <= i - window (pool_cache_blocks' layout); tokens and blocks share one
+    softmax over scale q.k, with 1 added to its denominator when unit_sink.  Query head h reads
+    key/value head h // (H / G).  Scores, softmax and the weighted sums are fp32.  Rows with
+    slot -1 are padding and left unwritten.  out [T, >= H Dv]."""
+    if _native(q):
+        torch.ops.akap_stream.pooled_window_attention(out, q, k_cache, v_cache, k_pool, v_pool,
+                                                      block_tables, q_start, positions, slots,
+                                                      float(scale), int(window), int(pool),
+                                                      bool(unit_sink))
+        return
+    T, H, D = q.shape
+    G, BS, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    rep = H // G
+    for b, (r0, r1) in enumerate(_row_sequences(T, q_start)):
+        for t in range(r0, r1):
+            if int(slots[t]) < 0:
+                continue
+            i = int(positions[t])
+            lo = max(0, i - window + 1) if window > 0 else 0
+            pos = torch.arange(lo, i + 1)
+            pages = block_tables[b][pos // BS].long()
+            K = k_cache[pages, :, pos % BS].float()            # [n, G, D]
+            V = v_cache[pages, :, pos % BS].float()
+            nb = (i - window + 1) // pool if (pool > 0 and window > 0 and i - window + 1 > 0) \
+                else 0
+            if nb > 0:
+                first = torch.arange(nb) * pool
+                pg = block_tables[b][first // BS].long()
+                K = torch.cat([k_pool[pg, :, (first % BS) // pool].float(), K])
+                V = torch.cat([v_pool[pg, :, (first % BS) // pool].float(), V])
+            for h in range(H):
+                s = (K[:, h // rep] @ q[t, h].float()) * scale
+                m = s.max()
+                if unit_sink:
+                    m = torch.clamp(m, min=0.0)
+                e = torch.exp(s - m)
+                den = e.sum() + (torch.exp(-m) if unit_sink else 0.0)
+                out[t, h * Dv:(h + 1) * Dv] = ((e / den) @ V[:, h // rep]).to(out.dtype)
+
+
+# ----------------------------------------------------------------------------- selective state space
+def conv_silu(out: torch.Tensor, proj: torch.Tensor, off: int, conv_w: torch.Tensor,
+              conv_b: torch.Tensor, state: torch.Tensor, seq_slot: torch.Tensor,
+              positions: torch.Tensor, q_start: Optional[torch.Tensor]) -> None:
+    """Causal per-channel convolution + silu over the columns [off, off + C) of proj [T, N]:
+    out[t, c] = silu(conv_b[c] + sum_j conv_w[c, j] u[t - (taps - 1 - j), c]) (fp32 [T, C]),
+    u the column of the sequence's earlier tokens: rows of this step, before them what an
+    earlier step left in state[slot] ([slots, taps - 1, C], proj's type, oldest first), zeros
+    before position 0.  After the step state[slot] holds the sequence's last taps - 1 inputs.
+    Sequences as in `retention`: rows [q_start[b], q_start[b + 1]) (None: one row each), slot =
+    seq_slot of the first row (-1: padding), fresh when that row has position 0.  conv_w
+    [C, taps], conv_b [C] fp32."""
+    if _native(proj):
+        torch.ops.akap_stream.conv_silu(out, proj, int(off), conv_w, conv_b, state, seq_slot,
+                                        positions, q_start)
+        return
+    C, taps = conv_w.shape
+    for r0, r1 in _row_sequences(proj.shape[0], q_start):
+        if r1 <= r0 or int(seq_slot[r0]) < 0:
+            continue
+        slot = int(seq_slot[r0])
+        prev = state[slot].float() if int(positions[r0]) > 0 else torch.zeros(taps - 1, C)
+        u = torch.cat([prev, proj[r0:r1, off:off + C].float()])      # [taps - 1 + n, C]
+        acc = conv_b.float()[None, :].repeat(r1 - r0, 1)
+        for j in range(taps):
+            acc = acc + conv_w[:, j].float()[None, :] * u[j:j + r1 - r0]
+        out[r0:r1] = torch.nn.functional.silu(acc)
+        if taps > 1:
+            state[slot] = u[-(taps - 1):].to(state.dtype)
+
+
+def selective_scan(y: torch.Tensor, xbc: torch.Tensor, proj: torch.Tensor, dt_off: int,
+                   dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor,
+                   state: torch.Tensor, seq_slot: torch.Tensor, positions: torch.Tensor,
+                   q_start: Optional[torch.Tensor], H: int, V: int, N: int, G: int) -> None:
+    """The state-space recurrence for the token rows of a step, fp32 throughout.  xbc [T, H V +
+    2 G N] (fp32) = [x | B | C]; dt_t,h = softplus(proj[t, dt_off + h] + dt_bias[h]) (no
+    clamp).  Per head h with group g = h // (H / G):  S <- exp(-exp(a_log[h]) dt) S + dt B_g
+    x_h^T (S is [N, V]),  y[t, h V : (h + 1) V] = S^T C_g + d_skip[h] x_h.  The state of a
+    sequence lives in state[slot, h] (fp32 [N, V]); sequences, slots and fresh starts as in
+    `retention`."""
+    if _native(xbc):
+        torch.ops.akap_stream.selective_scan(y, xbc, proj, int(dt_off), dt_bias, a_log, d_skip,
+                                             state, seq_slot, positions, q_start, H, V, N, G)
+        return
+    T = xbc.shape[0]
+    inner = H * V
+    x = xbc[:, :inner].float().view(T, H, V)
+    Bm = xbc[:, inner:inner + G * N].float().view(T, G, N).repeat_interleave(H // G, dim=1)
+    Cm = xbc[:, inner + G * N:inner + 2 * G * N].float().view(T, G, N).repeat_interleave(
+        H // G, dim=1)
+    dt = torch.nn.functional.softplus(proj[:, dt_off:dt_off + H].float() + dt_bias.float(),
+                                      threshold=30.0)
+    decay = torch.exp(-torch.exp(a_log.float())[None, :] * dt)            # [T, H]
+    for r0, r1 in _row_sequences(T, q_start):
+        if r1 <= r0 or int(seq_slot[r0]) < 0:
+            continue
+        slot = int(seq_slot[r0])
+        S = state[slot].clone() if int(positions[r0]) > 0 else torch.zeros(H, N, V)
+        for t in range(r0, r1):
+            S = decay[t][:, None, None] * S + dt[t][:, None, None] * Bm[t][:, :, None] \
+                * x[t][:, None, :]
+            y[t] = (torch.einsum("hnv,hn->hv", S, Cm[t]) + d_skip.float()[:, None] * x[t]
+                    ).reshape(inner)
+        state[slot] = S
+
+
+def gate_group_norm(out: torch.Tensor, y: torch.Tensor, gate: torch.Tensor, w: torch.Tensor,
+                    groups: int, eps: float) -> None:
+    """out = gnorm(y silu(gate)) w: y [T, n] fp32, gate [T, n] (a column slice of a projection),
+    the product RMS-normed in `groups` equal consecutive parts (each by its own root mean
+    square), times the fp32 weights w [n].  The gate comes before the norm.  fp32 arithmetic."""
+    if _native(y):
+        torch.ops.akap_stream.gate_group_norm(out, y, gate, w, int(groups), float(eps))
+        return
+    g = y.float() * torch.nn.functional.silu(gate.float())
+    out.copy_((_group_rms(g, groups, eps) * w.float()).to(out.dtype))
+
+
+# ----------------------------------------------------------------------------- sigmoid group routing
+def route_sigmoid(h: torch.Tensor, router: torch.Tensor, top: int, groups: int = 1,
+                  keep: int = 1, group_top: int = 2):
+    """Routing by sigmoid scores: s = sigmoid(router h) (fp32, from h's stored values); experts
+    form `groups` equal groups of neighbours, a group scores the sum of its `group_top` largest
+    s, only experts of the `keep` best groups can be chosen (ties: the lower index); the `top`
+    largest s among them win (ties: the lower index) and weigh their experts as they are.
+    Returns ids int32 [T, top] (by falling score) and weights fp32 [T, top].  router fp32
+    [E, d]."""
+    T, E = h.shape[0], router.shape[0]
+    ids = torch.empty(T, top, dtype=torch.int32, device=h.device)
+    w = torch.empty(T, top, dtype=torch.float32, device=h.device)
+    if _native(h):
+        torch.ops.akap_stream.route_sigmoid(ids, w, h, router, int(groups), int(keep),
+                                            int(group_top))
+        return ids, w
+    s = torch.sigmoid(h.float() @ router.float().T)
+    choice = s.clone()
+    per = E // groups
+    if groups > 1:
+        gs = s.view(T, groups, per).topk(min(group_top, per), dim=-1).values.sum(dim=-1)
+        best = torch.sort(gs, dim=-1, descending=True, stable=True).indices[:, :keep]
+        allowed = torch.zeros(T, groups, dtype=torch.bool).scatter_(1, best, True)
+        choice = choice.masked_fill(~allowed[:, :, None].expand(T, groups, per).reshape(T, E),
+                                    -1.0)
+    idx = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :top]
+    ids.copy_(idx)
+    w.copy_(s.gather(1, idx))
+    return ids, w
+
+
+def gated_act(gu: torch.Tensor, out: torch.Tensor, act: str = "silu",
+              ids: Optional[torch.Tensor] = None, w: Optional[torch.Tensor] = None,
+              experts: int = 1) -> None:
+    """out[t, e F + f] = w_e(t) act(gu[t, e 2F + f]) gu[t, e 2F + F + f] for gu [T, E 2F] = per
+    expert [gate | up]; act "silu" or "gelu_tanh" (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715
+    z^3)))); ids / w None: one plain gated layer (weight 1), else the routing weights as in
+    swiglu_routed.  fp32 arithmetic; both tensors may be column slices of wider rows."""
+    if act not in ("silu", "gelu_tanh"):
+        raise ValueError(f"gated_act: unknown activation {act!r}")
+    if _native(gu):
+        torch.ops.akap_stream.swiglu_routed(out, gu, ids, w, int(experts),
+                                            1 if act == "gelu_tanh" else 0)
+        return
+    T = gu.shape[0]
+    F_ = gu.shape[1] // (2 * experts)
+    g3 = gu.float().view(T, experts, 2, F_) if gu.is_contiguous() else \
+        gu.float().reshape(T, experts, 2, F_)
+    a = torch.nn.functional.silu(g3[:, :, 0]) if act == "silu" else \
+        torch.nn.functional.gelu(g3[:, :, 0], approximate="tanh")
+    r = a * g3[:, :, 1]
+    if ids is not None:
+        full = torch.zeros(T, experts, dtype=torch.float32)
+        full.scatter_(1, ids.long(), w)
+        r = r * full[:, :, None]
+    out.copy_(r.reshape(T, experts * F_).to(out.dtype))
