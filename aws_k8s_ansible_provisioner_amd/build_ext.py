@@ -219,18 +219,20 @@ def build_stream(force: bool = False, jobs: int = 8, log=None) -> str:
         if why:
             log(f"compile stream/{os.path.basename(src)} ({why})")
             todo.append((cmd, obj, digest))
-    ops_src = os.path.join(STREAM_SRC, "stream_ops.cpp")
-    ops_obj = os.path.join(BUILD, "stream_ops.cpp.o")
-    objs.append(ops_obj)
     incs = sum([["-I", i] for i in inc], [])
-    cmd = [HIPCC, *common, "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
-           "-DTORCH_EXTENSION_NAME=_C_stream", *incs, "-I", "/opt/rocm/include", "-x", "c++", "-c",
-           ops_src, "-o", ops_obj]
-    digest = _digest([ops_src] + headers, " ".join(cmd[:-3]) + f";torch={tv}")
-    why = "forced" if force else _stale(ops_obj, digest)
-    if why:
-        log(f"compile stream/stream_ops.cpp ({why})")
-        todo.append((cmd, ops_obj, digest))
+    # the op registrations: stream_ops.cpp defines the library, the other files add fragments
+    for ops_src in sorted(glob.glob(os.path.join(STREAM_SRC, "*.cpp"))):
+        base = os.path.basename(ops_src)
+        ops_obj = os.path.join(BUILD, ("" if base == "stream_ops.cpp" else "stream_") + base + ".o")
+        objs.append(ops_obj)
+        cmd = [HIPCC, *common, "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+               "-DTORCH_EXTENSION_NAME=_C_stream", *incs, "-I", "/opt/rocm/include", "-x", "c++",
+               "-c", ops_src, "-o", ops_obj]
+        digest = _digest([ops_src] + headers, " ".join(cmd[:-3]) + f";torch={tv}")
+        why = "forced" if force else _stale(ops_obj, digest)
+        if why:
+            log(f"compile stream/{base} ({why})")
+            todo.append((cmd, ops_obj, digest))
     with cf.ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
         list(ex.map(_compile, todo))
     out = os.path.join(PKG, "_C_stream.so")

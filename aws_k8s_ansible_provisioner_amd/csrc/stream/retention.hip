@@ -801,8 +801,12 @@ __global__ __launch_bounds__(256) void route_topk_kernel(int32_t* __restrict__ i
   for (int k = 0; k < top; ++k) wout[(size_t)t * top + k] *= inv;
 }
 
-// out[t, e F + f] = w_e(t) silu(gu[t, e 2F + f]) gu[t, e 2F + F + f]; ids null: weight 1
-template <typename T>
+// out[t, e F + f] = w_e(t) act(gu[t, e 2F + f]) gu[t, e 2F + F + f]; ids null: weight 1;
+// ACT 0: silu, 1: gelu in its tanh form
+__device__ __forceinline__ float gelu_tanhf(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+template <typename T, int ACT>
 __global__ __launch_bounds__(256) void swiglu_routed_kernel(T* __restrict__ out, int out_stride,
                                                             const T* __restrict__ gu, int gu_stride,
                                                             const int32_t* __restrict__ ids,
@@ -825,7 +829,7 @@ __global__ __launch_bounds__(256) void swiglu_routed_kernel(T* __restrict__ out,
     float r = 0.f;
     if (we != 0.f) {
       const float z = ldf(g + e * 2 * F + f);
-      r = we * z * sigmoidf(z) * ldf(g + e * 2 * F + F + f);
+      r = we * (ACT == 1 ? gelu_tanhf(z) : z * sigmoidf(z)) * ldf(g + e * 2 * F + F + f);
     }
     stf(o + c, r);
   }
@@ -979,15 +983,18 @@ void launch_route_topk(int32_t* ids, float* w, const void* h, int h_stride, cons
 
 void launch_swiglu_routed(void* out, int out_stride, const void* gu, int gu_stride,
                           const int32_t* ids, const float* w, int rows, int top, int E, int F,
-                          bool f32, hipStream_t s) {
+                          bool f32, int act, hipStream_t s) {
   if (rows <= 0) return;
   const size_t lds = (size_t)E * sizeof(float);
-  if (f32)
-    swiglu_routed_kernel<float><<<rows, 256, lds, s>>>((float*)out, out_stride, (const float*)gu,
-                                                       gu_stride, ids, w, top, E, F);
-  else
-    swiglu_routed_kernel<bf16><<<rows, 256, lds, s>>>((bf16*)out, out_stride, (const bf16*)gu,
-                                                      gu_stride, ids, w, top, E, F);
+#define AKAP_GA(TY, A)                                                                          \
+  swiglu_routed_kernel<TY, A><<<rows, 256, lds, s>>>((TY*)out, out_stride, (const TY*)gu,      \
+                                                     gu_stride, ids, w, top, E, F)
+  if (f32) {
+    if (act == 1) AKAP_GA(float, 1); else AKAP_GA(float, 0);
+  } else {
+    if (act == 1) AKAP_GA(bf16, 1); else AKAP_GA(bf16, 0);
+  }
+#undef AKAP_GA
 }
 
 }  // namespace akap_stream

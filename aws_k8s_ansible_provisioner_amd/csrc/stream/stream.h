@@ -250,8 +250,87 @@ void launch_route_topk(int32_t* ids, float* w, const void* h, int h_stride, cons
                        const float* bias, int rows, int d, int n, int top, bool f32,
                        hipStream_t s);
 // ids null: every weight is 1 (E = 1: a plain gated activation of [gate | up] rows)
+// act 0: silu on the gate, 1: the tanh form of gelu
 void launch_swiglu_routed(void* out, int out_stride, const void* gu, int gu_stride,
                           const int32_t* ids, const float* w, int rows, int top, int E, int F,
-                          bool f32, hipStream_t s);
+                          bool f32, int act, hipStream_t s);
+
+// ---- several residual streams, state-space mixer, sigmoid group routing (hyper.hip) -----------
+// xs [rows, S, d] fp32 in place: every stream from the old ones, xs_r <- sum_s mix[s, r] xs_s +
+// w_out[r] (ya + yb + bias) (fresh: every stream <- fresh row); then u = sum_s w_in[s] xs_s and
+// out = rmsnorm(u) * norm_w.  ya / yb rows of bf16 or fp32, each may be null.  S <= 8.
+void launch_hyper_step(void* out, bool out_f32, int out_stride, float* xs, const float* fresh,
+                       const void* ya, bool ya_f32, int ya_stride, const void* yb, bool yb_f32,
+                       int yb_stride, const float* bias, const float* mix, const float* w_out,
+                       const float* w_in, const float* norm_w, int rows, int S, int d, float eps,
+                       hipStream_t s);
+void launch_softcap(void* x, bool f32, size_t n, float cap, hipStream_t s);
+// out = gnorm(y * silu(gate)) * w over `groups` equal parts of the n columns
+void launch_gate_group_norm(void* out, int out_stride, const float* y, const void* gate,
+                            int gate_stride, const float* w, bool f32, int rows, int n,
+                            int groups, float eps, hipStream_t s);
+void launch_route_sigmoid(int32_t* ids, float* w, const void* h, int h_stride, bool f32,
+                          const float* router, int rows, int d, int E, int top, int groups,
+                          int keep, int group_top, hipStream_t s);
+// causal per-channel convolution + silu of columns [off, off + C) of proj, then the sequences'
+// last taps - 1 inputs to their slots; B sequences (q_start null: B = T, one row each)
+void launch_conv_silu(float* out, const void* proj, int proj_stride, int off, bool f32,
+                      void* state, const float* w, const float* b, const int32_t* seq_slot,
+                      const int64_t* positions, const int32_t* q_start, int T, int B, int C,
+                      int taps, hipStream_t s);
+// state rows a thread of the scan keeps in registers (at most 64)
+int selective_scan_rows(int V, int N);
+void launch_selective_scan(float* y, const float* xbc, const void* proj, int proj_stride,
+                           int dt_off, bool f32, const float* dt_bias, const float* a_log,
+                           const float* d_skip, float* state, const int32_t* seq_slot,
+                           const int64_t* positions, const int32_t* q_start, int T, int B, int H,
+                           int V, int N, int G, hipStream_t s);
+
+// ---- window + pooled blocks attention (pooled_attention.hip) -----------------------------------
+struct RopeCacheParams {
+  const void* proj;      // [T, N] fused projection rows
+  int proj_stride;
+  void* q_out;           // [T, H, D]
+  void* k_cache;         // [NB, G, BS, D]
+  void* v_cache;         // [NB, G, BS, Dv]
+  const int64_t* positions;
+  const int64_t* slots;
+  const float* cos_sin;  // [max_pos, rot_dims] = [cos | sin], or null
+  const float* bias;     // [N] laid out like proj's columns, or null
+  int max_pos, rot_dims;
+  int T, H, G, D, Dv, BS, q_off, k_off, v_off;
+  int64_t num_slots;
+};
+void launch_bias_rope_cache(const RopeCacheParams& p, bool f32, hipStream_t s);
+
+struct PoolParams {
+  const void* k_cache;
+  const void* v_cache;
+  float* k_pool;         // [NB, G, PS, D]
+  float* v_pool;
+  const int64_t* positions;
+  const int64_t* slots;
+  const int32_t* block_tables;
+  const int32_t* q_start;   // [B + 1] or null
+  int max_blocks, T, B, G, D, Dv, BS, PS, pool;
+};
+void launch_pool_cache_blocks(const PoolParams& p, bool f32, hipStream_t s);
+
+struct PoolAttnParams {
+  void* out;             // rows of out_stride; head h at columns [h Dv, (h + 1) Dv)
+  int out_stride;
+  const void* q;         // [T, H, D]
+  const void* k_cache;
+  const void* v_cache;
+  const float* k_pool;   // or null (pool 0)
+  const float* v_pool;
+  const int32_t* block_tables;
+  const int32_t* q_start;
+  const int64_t* positions;
+  const int64_t* slots;
+  float scale;
+  int max_blocks, T, B, H, G, D, Dv, BS, PS, window, pool, unit_sink;
+};
+void launch_pooled_window_attention(const PoolAttnParams& p, bool f32, hipStream_t s);
 
 }  // namespace akap_stream

@@ -974,7 +974,8 @@ void route_topk(Tensor ids, Tensor w, Tensor h, Tensor router, std::optional<Ten
 }
 
 void swiglu_routed(Tensor out, Tensor gu, std::optional<Tensor> ids, std::optional<Tensor> w,
-                   int64_t experts) {
+                   int64_t experts, int64_t act) {
+  TORCH_CHECK(act == 0 || act == 1, "swiglu_routed: act is 0 (silu) or 1 (gelu, tanh form)");
   CHECK_GPU(out); CHECK_GPU(gu); CHECK_LAST_CONTIG(out); CHECK_LAST_CONTIG(gu);
   TORCH_CHECK(out.scalar_type() == gu.scalar_type() && out.dim() == 2 && gu.dim() == 2 &&
                   out.size(0) == gu.size(0) && experts >= 1 && gu.size(1) == 2 * out.size(1) &&
@@ -993,7 +994,8 @@ void swiglu_routed(Tensor out, Tensor gu, std::optional<Tensor> ids, std::option
   const c10::DeviceGuard g(gu.device());
   akap_stream::launch_swiglu_routed(out.data_ptr(), (int)out.stride(0), gu.data_ptr(),
                                     (int)gu.stride(0), ip, wp, (int)T, top, (int)experts,
-                                    (int)(out.size(1) / experts), is_f32(gu, "gu"), cur_stream());
+                                    (int)(out.size(1) / experts), is_f32(gu, "gu"), (int)act,
+                                    cur_stream());
 }
 
 }  // namespace
@@ -1064,7 +1066,8 @@ TORCH_LIBRARY(akap_stream, m) {
         "Tensor block_tables, Tensor seq_lens, Tensor positions, Tensor? talk, Tensor? gate, "
         "float scale, Tensor(b!) ws_ml, Tensor(c!) ws_o, int num_parts) -> ()");
   m.def("route_topk(Tensor(a!) ids, Tensor(b!) w, Tensor h, Tensor router, Tensor? bias) -> ()");
-  m.def("swiglu_routed(Tensor(a!) out, Tensor gu, Tensor? ids, Tensor? w, int experts) -> ()");
+  m.def("swiglu_routed(Tensor(a!) out, Tensor gu, Tensor? ids, Tensor? w, int experts, "
+        "int act=0) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(akap_stream, CUDA, m) {

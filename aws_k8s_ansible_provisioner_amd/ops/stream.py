@@ -1161,14 +1161,15 @@ def conv_silu(out: torch.Tensor, proj: torch.Tensor, off: int, conv_w: torch.Ten
         if r1 <= r0 or int(seq_slot[r0]) < 0:
             continue
         slot = int(seq_slot[r0])
-        prev = state[slot].float() if int(positions[r0]) > 0 else torch.zeros(taps - 1, C)
+        prev = state[slot, :taps - 1].float() if int(positions[r0]) > 0 \
+            else torch.zeros(taps - 1, C)
         u = torch.cat([prev, proj[r0:r1, off:off + C].float()])      # [taps - 1 + n, C]
         acc = conv_b.float()[None, :].repeat(r1 - r0, 1)
         for j in range(taps):
             acc = acc + conv_w[:, j].float()[None, :] * u[j:j + r1 - r0]
         out[r0:r1] = torch.nn.functional.silu(acc)
         if taps > 1:
-            state[slot] = u[-(taps - 1):].to(state.dtype)
+            state[slot, :taps - 1] = u[-(taps - 1):].to(state.dtype)
 
 
 def selective_scan(y: torch.Tensor, xbc: torch.Tensor, proj: torch.Tensor, dt_off: int,

@@ -288,3 +288,69 @@ def forward(cfg, w, tokens, store=None):
     if cap:
         logits = cap * torch.tanh(logits / cap)
     return logits, torch.stack(after)
+
+
+# ----------------------------------------------------------------------------- test models
+def random_weights(cfg, seed=0):
+    """Random weights under the checkpoint's names, values a bf16 file can hold (bf16 tensors).
+    Norm weights sit around zero, stream weights around an identity, decays and step sizes in a
+    range where the state neither dies at once nor stays for ever."""
+    g = torch.Generator().manual_seed(seed)
+    d, S = int(cfg["width"]), int(cfg.get("streams") or 0)
+
+    def rnd(*shape, s=1.0, mean=0.0):
+        return (torch.randn(*shape, generator=g) * s + mean).to(torch.bfloat16)
+
+    w = {"embed": rnd(int(cfg["vocab"]), d), "final.norm": rnd(d, s=0.2)}
+    for i, ly in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        m = ly["mixer"]
+        w[p + "norm1"] = rnd(d, s=0.2)
+        subs = ["hc1"]
+        if ly["type"] == "attention":
+            H, G, D, Dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
+            for name, rows in (("q", H * D), ("k", G * D), ("v", G * Dv)):
+                w[p + "mix." + name] = rnd(rows, d, s=d ** -0.5)
+                w[p + "mix." + name + ".b"] = rnd(rows, s=0.3)
+            w[p + "mix.o"] = rnd(d, H * Dv, s=(H * Dv) ** -0.5)
+            w[p + "mix.o.b"] = rnd(d, s=0.3)
+        else:
+            H, V, N, G = int(m["heads"]), int(m["vdim"]), int(m["state"]), int(m["groups"])
+            inner, C = H * V, H * V + 2 * G * N
+            w[p + "mix.in"] = rnd(2 * inner + 2 * G * N + H, d, s=d ** -0.5)
+            w[p + "mix.conv"] = rnd(C, int(m["conv"]), s=0.5)
+            w[p + "mix.conv.b"] = rnd(C, s=0.2)
+            w[p + "mix.dt_bias"] = rnd(H, s=1.0, mean=-1.0)
+            w[p + "mix.A_log"] = rnd(H, s=0.7, mean=-0.5)
+            w[p + "mix.D"] = rnd(H, s=0.3, mean=1.0)
+            w[p + "mix.norm"] = rnd(inner, s=0.2, mean=1.0)
+            w[p + "mix.o"] = rnd(d, inner, s=inner ** -0.5)
+        ml = ly.get("mlp")
+        if ml is not None:
+            w[p + "norm2"] = rnd(d, s=0.2)
+            subs.append("hc2")
+
+            def gated_w(q, ff):
+                w[q + "gate"] = rnd(ff, d, s=d ** -0.5)
+                w[q + "up"] = rnd(ff, d, s=d ** -0.5)
+                w[q + "down"] = rnd(d, ff, s=ff ** -0.5)
+
+            if ml["kind"] == "dense":
+                gated_w(p + "mlp.", int(ml["ff"]))
+            else:
+                w[p + "mlp.router"] = rnd(int(ml["router"]["experts"]), d, s=2 * d ** -0.5)
+                for e in range(int(ml["router"]["experts"])):
+                    gated_w(p + f"mlp.e{e}.", int(ml["expert"]["ff"]))
+                if ml.get("shared"):
+                    gated_w(p + "mlp.shared.", int(ml["shared"]["ff"]))
+        if S:
+            for name in subs:
+                w[p + name + ".in"] = rnd(S, s=0.3, mean=1.0 / S)
+                w[p + name + ".out"] = rnd(S, s=0.3, mean=0.8)
+                w[p + name + ".mix"] = (torch.eye(S) + 0.15 * torch.randn(S, S, generator=g)
+                                        ).to(torch.bfloat16)
+    return w
+
+
+def as_f64(weights):
+    return {k: v.to(F64) for k, v in weights.items()}

@@ -1,0 +1,221 @@
+"""Mudepel on the HIP kernels: every new kernel against the PyTorch version of the same op (fp32
+and bf16 storage, odd sizes), then the engine -- mixed steps, hipGraph decode, a small page and
+slot pool -- against the float64 oracle (tests/mudepel_oracle.py), and greedy generation
+through LLMEngine.generate."""
+import pytest
+import torch
+
+import mudepel_oracle as oracle
+from bidetar_harness import engine, rel_err, replay, tokens, write_model
+from aws_k8s_ansible_provisioner_amd.ops import stream as sops
+
+pytestmark = pytest.mark.gpu
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+TOL = {"float32": 3e-4, "bfloat16": 0.3}
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def close(a, b, dtype, scale=1.0):
+    tol = 3e-5 if dtype == "float32" else 2e-2
+    torch.testing.assert_close(a.float().cpu(), b.float().cpu(), rtol=tol, atol=tol * scale)
+
+
+def both(fn):
+    """fn(device) on the CPU and on the GPU; returns the two results."""
+    return fn("cpu"), fn("cuda")
+
+
+# ------------------------------------------------------------------ kernels against their ops
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("S,d", [(1, 24), (3, 200), (4, 2048), (8, 514), (2, 8192)])
+def test_hyper_step_kernel(dtype, S, d):
+    g, dt = gen(S * d), DT[dtype]
+    T = 5
+    xs0 = torch.randn(T, S, d, generator=g)
+    ya = torch.randn(T, d + 8, generator=g).to(dt)[:, :d]
+    yb = torch.randn(T, d, generator=g)
+    bias = torch.randn(d, generator=g)
+    mix = torch.eye(S) + 0.3 * torch.randn(S, S, generator=g)
+    wo, wi = torch.randn(S, generator=g), torch.randn(S, generator=g)
+    nw = 1 + 0.3 * torch.randn(d, generator=g)
+    e = torch.randn(T, d, generator=g)
+    for a, b, bb, fresh in ((ya, None, None, None), (ya, yb, bias, None), (None, yb, None, None),
+                            (None, None, None, e)):
+        def run(dev):
+            mv = lambda t: None if t is None else t.to(dev)  # noqa: E731
+            xs = xs0.clone().to(dev)
+            o = torch.zeros(T, d, dtype=dt, device=dev)
+            sops.hyper_step(xs, mv(a), mv(b), mv(bb), mv(mix), mv(wo), mv(wi), mv(nw), 1e-6, o,
+                            fresh=mv(fresh))
+            return xs, o
+        c, n = both(run)
+        close(n[0], c[0], "float32", scale=4.0)
+        close(n[1], c[1], dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_softcap_and_gated_act_kernels(dtype):
+    g, dt = gen(3), DT[dtype]
+    x = (20 * torch.randn(7, 333, generator=g)).to(dt)
+    c, n = both(lambda dev: sops.softcap_(x.clone().to(dev), 12.5))
+    close(n, c, dtype, scale=12.5)
+    E, F_, T = 5, 24, 9
+    gu = (2 * torch.randn(T, E * 2 * F_ + 6, generator=g)).to(dt)
+    ids = torch.stack([torch.randperm(E, generator=g)[:2] for _ in range(T)]).int()
+    w = torch.rand(T, 2, generator=g)
+    for act in ("silu", "gelu_tanh"):
+        def run(dev):
+            o = torch.zeros(T, E * F_ + 4, dtype=dt, device=dev)
+            sops.gated_act(gu.to(dev)[:, :E * 2 * F_], o[:, :E * F_], act, ids.to(dev), w.to(dev), E)
+            o2 = torch.zeros(T, E * F_, dtype=dt, device=dev)
+            sops.gated_act(gu.to(dev)[:, :E * 2 * F_], o2, act, None, None, E)
+            return o, o2
+        c, n = both(run)
+        close(n[0], c[0], dtype, scale=4.0)
+        close(n[1], c[1], dtype, scale=4.0)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n,groups", [(48, 3), (512, 1), (640, 5), (4096, 8)])
+def test_gate_group_norm_kernel(dtype, n, groups):
+    g, dt = gen(n), DT[dtype]
+    T = 6
+    y = 3 * torch.randn(T, n, generator=g)
+    gate = torch.randn(T, n + 16, generator=g).to(dt)
+    w = 1 + 0.2 * torch.randn(n, generator=g)
+
+    def run(dev):
+        o = torch.zeros(T, n, dtype=dt, device=dev)
+        sops.gate_group_norm(o, y.to(dev), gate.to(dev)[:, 8:8 + n], w.to(dev), groups, 1e-5)
+        return o
+    c, nn = both(run)
+    close(nn, c, dtype, scale=3.0)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("E,top,groups,keep,d", [(16, 4, 4, 2, 160), (6, 2, 3, 2, 40),
+                                                 (8, 8, 1, 1, 64), (12, 4, 4, 2, 1024),
+                                                 (5, 1, 5, 3, 33), (64, 6, 8, 4, 256)])
+def test_route_sigmoid_kernel(dtype, E, top, groups, keep, d):
+    g, dt = gen(E * d), DT[dtype]
+    T = 40
+    h = torch.randn(T, d, generator=g).to(dt)
+    router = (torch.randn(E, d, generator=g) * 2 * d ** -0.5)
+    (ci, cw), (ni, nw) = both(lambda dev: sops.route_sigmoid(h.to(dev), router.to(dev), top, groups,
+                                                            keep, 2))
+    # a choice may differ only where two scores are within rounding of each other
+    same = (ci == ni.cpu()).all(dim=1)
+    assert same.float().mean() > 0.9
+    close(nw[same], cw[same], "float32")
+
+
+def _conv_scan_case(dtype, H, V, N, G, taps, dev, steps, g, slots=3):
+    """Run `steps` (each a list of (slot, first position, rows)) through convolution, scan and
+    gate; returns the outputs of all steps and the final states."""
+    dt = DT[dtype]
+    inner, C = H * V, H * V + 2 * G * N
+    rows = 2 * inner + 2 * G * N + H + 5
+    cw = (0.5 * torch.randn(C, taps, generator=g)).to(dev)
+    cb = (0.2 * torch.randn(C, generator=g)).to(dev)
+    dtb = (torch.randn(H, generator=g) - 1).to(dev)
+    alog = (0.7 * torch.randn(H, generator=g) - 0.5).to(dev)
+    dsk = (1 + 0.3 * torch.randn(H, generator=g)).to(dev)
+    cst = torch.full((slots, max(1, taps - 1), C), 7.0, dtype=dt, device=dev)   # stale contents
+    st = torch.full((slots, H, N, V), 7.0, device=dev)
+    outs = []
+    for step in steps:
+        T = sum(n for _, _, n in step)
+        proj = torch.randn(T, rows, generator=g).to(dt).to(dev)
+        slot = torch.cat([torch.full((n,), s, dtype=torch.int32) for s, _, n in step]).to(dev)
+        pos = torch.cat([torch.arange(p, p + n) for _, p, n in step]).to(dev)
+        single = all(n == 1 for _, _, n in step)
+        qs = None
+        if not single:
+            qs = torch.tensor([0] + [n for _, _, n in step]).cumsum(0).int().to(dev)
+        xbc = torch.zeros(T, C, device=dev)
+        sops.conv_silu(xbc, proj, inner, cw, cb, cst, slot, pos, qs)
+        y = torch.zeros(T, inner, device=dev)
+        sops.selective_scan(y, xbc, proj, inner + C, dtb, alog, dsk, st, slot, pos, qs, H, V, N, G)
+        outs += [xbc, y]
+    return outs, cst, st
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,V,N,G,taps", [(4, 32, 16, 4, 3), (3, 16, 8, 1, 2), (2, 64, 128, 2, 4),
+                                          (6, 48, 20, 3, 3), (1, 128, 64, 1, 1), (8, 8, 16, 8, 5)])
+def test_conv_and_scan_kernels(dtype, H, V, N, G, taps):
+    # a prompt in portions (one shorter than the taps), a mixed step, single rows, a slot used
+    # again from position 0 on top of stale contents, a padding row (slot -1)
+    steps = [[(0, 0, 37), (1, 0, 2)], [(1, 2, 1), (0, 37, 1)], [(0, 38, 19), (1, 3, 2), (2, 0, 1)],
+             [(2, 1, 1), (-1, 0, 1), (1, 5, 1)], [(1, 0, 21)]]
+    c = _conv_scan_case(dtype, H, V, N, G, taps, "cpu", steps, gen(H * V + N))
+    n = _conv_scan_case(dtype, H, V, N, G, taps, "cuda", steps, gen(H * V + N))
+    for i, (a, b) in enumerate(zip(c[0], n[0])):
+        if i // 2 == 3:          # the padding row is left unwritten
+            a, b = a[[0, 2]], b[[0, 2]]
+        close(b, a, "float32", scale=8.0)
+    close(n[1], c[1], dtype)
+    close(n[2], c[2], "float32", scale=8.0)
+
+
+def _attention_case(dtype, H, G, D, Dv, rot, window, pool, BS, dev, steps, g, sink=True):
+    dt = DT[dtype]
+    NB = 24
+    N = H * D + G * (D + Dv) + 3
+    kc = torch.zeros(NB, G, BS, D, dtype=dt, device=dev)
+    vc = torch.zeros(NB, G, BS, Dv, dtype=dt, device=dev)
+    PS = sops.pool_slots(BS, pool)
+    kp = torch.full((NB, G, max(PS, 1), D), 5.0, device=dev) if pool else None
+    vp = torch.full((NB, G, max(PS, 1), Dv), 5.0, device=dev) if pool else None
+    cs = sops.rotary_table_yarn(512, rot, 1000.0, {"factor": 4.0, "original": 64, "fast": 8.0,
+                                                   "slow": 1.0}).to(dev) if rot else None
+    bias = (0.3 * torch.randn(N, generator=g)).to(dev)
+    # two sequences on interleaved pages in a scrambled order
+    perm = torch.randperm(NB, generator=g).int()
+    bt_all = torch.stack([perm[:NB // 2], perm[NB // 2:]])
+    outs = []
+    for step in steps:
+        T = sum(n for _, _, n in step)
+        proj = torch.randn(T, N, generator=g).to(dt).to(dev)
+        seqs = [s for s, _, _ in step]
+        pos = torch.cat([torch.arange(p, p + n) for _, p, n in step])
+        sq = torch.cat([torch.full((n,), s) for s, _, n in step])
+        slots = torch.where(sq >= 0, bt_all[sq.clamp(min=0), pos // BS].long() * BS + pos % BS,
+                            torch.tensor(-1))
+        bt = bt_all[torch.tensor(seqs).clamp(min=0)].to(dev)
+        single = all(n == 1 for _, _, n in step)
+        qs = None if single else torch.tensor([0] + [n for _, _, n in step]).cumsum(0).int().to(dev)
+        q = torch.zeros(T, H, D, dtype=dt, device=dev)
+        sops.bias_rope_cache(proj, q, kc, vc, pos.to(dev), slots.to(dev), cs, bias, H, G, D, Dv,
+                             0, H * D, H * D + G * D)
+        if pool:
+            sops.pool_cache_blocks(kc, vc, kp, vp, pos.to(dev), slots.to(dev), bt, qs, pool)
+        o = torch.zeros(T, H * Dv + 2, dtype=dt, device=dev)
+        sops.pooled_window_attention(o, q, kc, vc, kp, vp, bt, qs, pos.to(dev), slots.to(dev),
+                                     0.3, window, pool, sink)
+        keep = (slots >= 0)
+        outs += [q[keep.to(dev)], o[keep.to(dev)]]
+    return outs, kc, vc
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,G,D,Dv,rot,window,pool,BS", [
+    (6, 3, 64, 64, 32, 44, 12, 32), (4, 2, 32, 16, 16, 24, 8, 32), (3, 1, 20, 36, 8, 10, 3, 16),
+    (8, 2, 128, 128, 64, 50, 48, 32), (2, 2, 8, 8, 0, 0, 0, 32), (4, 4, 16, 24, 16, 33, 0, 32),
+    (5, 5, 12, 7, 12, 7, 20, 16)])
+def test_attention_kernels(dtype, H, G, D, Dv, rot, window, pool, BS):
+    # prompts in portions across pages and pooled blocks, a mixed step, single rows, a padding row
+    steps = [[(0, 0, 70), (1, 0, 3)], [(1, 3, 1), (0, 70, 1)], [(0, 71, 59), (1, 4, 30)],
+             [(0, 130, 1), (-1, 0, 1), (1, 34, 1)], [(1, 35, 61)], [(0, 131, 1), (1, 96, 1)]]
+    for sink in (True, False):
+        c = _attention_case(dtype, H, G, D, Dv, rot, window, pool, BS, "cpu", steps, gen(H * D),
+                            sink)
+        n = _attention_case(dtype, H, G, D, Dv, rot, window, pool, BS, "cuda", steps, gen(H * D),
+                            sink)
+        for a, b in zip(c[0], n[0]):
+            close(b, a, dtype, scale=2.0)
+        close(n[1], c[1], dtype, scale=2.0)
+        close(n[2], c[2], dtype, scale=2.0)
