@@ -76,6 +76,8 @@ class StreamLayerWeights:
     w_up: Optional[torch.Tensor] = None       # dense [2 ff, d] = [gate | up]; routed: per expert
     w_down: Optional[torch.Tensor] = None     # [gate | up] then the shared one; [d, sum of ffs]
     router: Optional[torch.Tensor] = None     # fp32 [E, d]
+    w_down_e: Optional[torch.Tensor] = None   # [E, d, F]: the routed experts' down-projections,
+                                              # made on first use
 
 
 class MudepelLM:
@@ -262,6 +264,8 @@ class MudepelLM:
                 raise ValueError(f"{name}: checkpoint shape {tuple(src.shape)} does not fit the "
                                  f"config (wanted {tuple(dst.shape)})")
             dst.copy_(src.to(dst.dtype))
+        for lw in self.layers:
+            lw.w_down_e = None
         self._derive()
 
     @property
@@ -269,7 +273,7 @@ class MudepelLM:
         return True
 
     def weight_bytes(self) -> int:
-        skip = ("cos_sin", "norm1p", "norm2p", "spec", "hc1", "hc2")
+        skip = ("cos_sin", "norm1p", "norm2p", "spec", "hc1", "hc2", "w_down_e")
         seen = [self.embed, self.final_norm]
         for lw in self.layers:
             seen += [getattr(lw, f.name) for f in dataclasses.fields(lw)
@@ -400,6 +404,13 @@ class MudepelLM:
         sops.gate_group_norm(g, y, proj[:, :inner], lw.gnorm, m.norm_groups, self.cfg.rms_eps)
         return self._linear(g, lw.w_o)
 
+    def _grouped_ok(self, h2: torch.Tensor, ff: int) -> bool:
+        """Can the core library's grouped expert GEMMs run this layer (bf16 on the GPU, the
+        library loaded -- a replay engine that returns logits alone runs without it --, both
+        reduction depths multiples of 64)?"""
+        return (h2.is_cuda and self.dtype == torch.bfloat16 and ops.native_loaded()
+                and h2.shape[1] % 64 == 0 and ff % 64 == 0)
+
     def _feed_forward(self, lw: StreamLayerWeights, h2: torch.Tensor, small: bool):
         """(output in the activation type or None, fp32 output or None) of the feed-forward."""
         ml = lw.spec.mlp
@@ -430,7 +441,16 @@ class MudepelLM:
             sops.gated_act(gu, u, "silu")
             return F.linear(u, lw.w_down[:, e * F_:(e + 1) * F_])
 
-        routed = routed_sorted(h2, ids, w, E, E, expert)
+        if self._grouped_ok(h2, F_):
+            # prompt-sized batches on an engine that has the core library: the framework's
+            # grouped expert GEMMs (device-side sort and tile map, silu gate in the epilogue, no
+            # host round trip); they take the down-projections per expert, [E, d, F]
+            if lw.w_down_e is None:
+                lw.w_down_e = lw.w_down[:, :E * F_].reshape(d, E, F_).permute(1, 0, 2).contiguous()
+            routed = ops.fused_moe(h2, lw.w_up[:E * 2 * F_].view(E, 2 * F_, d), lw.w_down_e, w,
+                                   ids)
+        else:
+            routed = routed_sorted(h2, ids, w, E, E, expert)
         shared = None
         if Fs:
             gu = self._linear(h2, lw.w_up[E * 2 * F_:])

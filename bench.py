@@ -89,7 +89,7 @@ def parse():
                          "kernel table")
     ap.add_argument("--profile-steps", type=int, default=0,
                     help="extra untimed waves run after timing (for rocprofv3 captures)")
-    ap.add_argument("--compare-design", default=None, choices=["bidetar", "puputar", "sazepel"],
+    ap.add_argument("--compare-design", default=None, choices=["bidetar", "puputar", "sazepel", "mudepel"],
                     help="instead of the serving wave: prefill and decode throughput of this "
                          "design at real layer sizes (random weights) beside the closest "
                          "existing model of equal size; prints one JSON line with the table")
@@ -112,6 +112,11 @@ COMPARE_SETS = {
     # and the one with routed experts
     "sazepel": [("sazepel-w2048", "bidetar-w2048"), ("sazepel-w4096", "bidetar-w4096"),
                 ("puputar-w2048-moe", None)],
+    # state-space layers + windowed attention over pooled blocks + routed experts on several
+    # residual streams beside the framework's other hybrid of a recurrent state, an attention
+    # and routed experts at the same width and depth, and the dense fp32-stream design
+    "mudepel": [("mudepel-w2048", "sazepel-w2048"), ("mudepel-w4096", "sazepel-w4096"),
+                ("bidetar-w2048", None)],
 }
 
 

@@ -354,3 +354,42 @@ def random_weights(cfg, seed=0):
 
 def as_f64(weights):
     return {k: v.to(F64) for k, v in weights.items()}
+
+
+def att_layer(heads, kv_heads, dim, vdim, scale, window=0, pool=0, rot_dims=None, base=100.0,
+              yarn=None, mlp=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale,
+         "rot": {"dims": dim if rot_dims is None else rot_dims, "base": base, "scaling": yarn}}
+    if window:
+        m["mask"] = {"size": window, "pool": pool}
+    return {"type": "attention", "mixer": m, "mlp": mlp}
+
+
+def ssm_layer(heads, vdim, state, groups, conv=4, norm_groups=1, mlp=None):
+    return {"type": "mamba2", "mlp": mlp,
+            "mixer": {"heads": heads, "vdim": vdim, "state": state, "groups": groups, "conv": conv,
+                      "norm_groups": norm_groups}}
+
+
+def dense(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def routed(experts, top, ff, count=1, keep=1, shared=0):
+    ml = {"kind": "moe", "expert": {"ff": ff},
+          "router": {"experts": experts, "top": top, "groups": {"count": count, "keep": keep}}}
+    if shared:
+        ml["shared"] = {"ff": shared}
+    return ml
+
+
+def make_config(width, vocab, layers, streams=2, eps=1e-5, softcap=12.0, loop=None):
+    cfg = {"architecture": "Mudepel", "layers": layers, "norm": {"eps": eps}, "vocab": vocab,
+           "width": width}
+    if streams:
+        cfg["streams"] = streams
+    if softcap:
+        cfg["logit_softcap"] = softcap
+    if loop:
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return cfg

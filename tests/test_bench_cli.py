@@ -110,7 +110,8 @@ def test_bench_gpus_n_without_launcher_starts_n_ranks():
 
 @pytest.mark.parametrize("design,models", [("bidetar", "tiny-bidetar,tiny-llama"),
                                            ("puputar", "tiny-puputar,tiny-bidetar"),
-                                           ("sazepel", "tiny-sazepel,tiny-bidetar")])
+                                           ("sazepel", "tiny-sazepel,tiny-bidetar"),
+                                           ("mudepel", "tiny-mudepel,tiny-sazepel")])
 def test_bench_compare_design_option(design, models):
     """--compare-design prints one JSON line with prefill and decode throughput per model and
     leaves the default output alone."""

@@ -219,3 +219,162 @@ def test_attention_kernels(dtype, H, G, D, Dv, rot, window, pool, BS):
             close(b, a, dtype, scale=2.0)
         close(n[1], c[1], dtype, scale=2.0)
         close(n[2], c[2], dtype, scale=2.0)
+
+
+# ------------------------------------------------------------------ the engine on the GPU
+from test_mudepel import OTHER, base_config  # noqa: E402
+
+
+def check(got, want, dtype, names=None):
+    for n in names or got:
+        e = rel_err(got[n], want[n])
+        if dtype == "float32":
+            assert e.max().item() < TOL[dtype], \
+                f"{n}: position {int(e.argmax())} off by {e.max().item():.2e}"
+        else:   # small widths: bf16 rounding is large and a close routing call flips a position
+            assert e.median().item() < 0.15, f"{n}: median error {e.median().item():.2e}"
+
+
+@pytest.fixture(scope="module")
+def model(tmp_path_factory):
+    cfg = base_config()
+    W = oracle.random_weights(cfg, seed=2)
+    W64 = oracle.as_f64(W)
+    reqs = {"a": tokens(75, cfg["vocab"], 1), "b": tokens(41, cfg["vocab"], 2),
+            "c": tokens(23, cfg["vocab"], 3), "d": tokens(1, cfg["vocab"], 4),
+            "e": tokens(64, cfg["vocab"], 5)}
+    want = {n: oracle.forward(cfg, W64, t)[0] for n, t in reqs.items()}
+    return cfg, W, write_model(tmp_path_factory.mktemp("mudepel_gpu"), cfg, W), reqs, want
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("eager", [False, True])
+def test_schedules(model, dtype, eager):
+    _, _, path, reqs, want = model
+    eng = engine(path, dtype=dtype, device="cuda", eager=eager)
+    assert eager or eng.runner.graphs, "decode hipGraphs were not captured"
+    one = {"a": reqs["a"]}
+    check(replay(eng, reqs, [[(n, len(t))] for n, t in reqs.items()]), want, dtype)
+    check(replay(eng, one, [[("a", 40)]] + [[("a", 1)]] * 35), want, dtype)
+    check(replay(eng, one, [[("a", s)] for s in [3, 2, 7, 2, 19, 2, 5, 33, 2]]), want, dtype)
+    sched = [[("a", 30), ("b", 2), ("c", 1)],
+             [("a", 1), ("b", 20), ("c", 22), ("d", 1)],
+             [("a", 1), ("b", 1), ("e", 33)],
+             [("a", 1), ("b", 1)],
+             [("b", 17), ("e", 1)],
+             [("a", 42), ("e", 30)]]
+    check(replay(eng, reqs, sched), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_small_pool_is_used_again(model, dtype):
+    _, _, path, reqs, want = model
+    eng = engine(path, dtype=dtype, max_tokens=160, max_seqs=2, device="cuda")
+    many = {f"{n}{i}": reqs[n] for i in range(2) for n in ("b", "c", "e")}
+    many["a"] = reqs["a"]
+    sched = [[("b0", 41), ("c0", 23)], [("e0", 64), ("c1", 22)], [("c1", 1)],
+             [("a", 75), ("b1", 41)], [("e1", 10)], [("e1", 54)]]
+    for _ in range(2):  # graphs replayed again over pages and slots that changed owners
+        check(replay(eng, many, sched), {k: want[k[0]] for k in many}, dtype)
+    assert eng.sched.num_free_blocks() == 5 and eng.sched.num_free_tail_slots == 2
+
+
+def test_long_decode_through_graphs(tmp_path):
+    """Decoding while the window and its pooled blocks pass over decoded tokens, the states and
+    convolution inputs carried by the captured graphs."""
+    cfg = oracle.make_config(width=64, vocab=37, streams=2, layers=[
+        oracle.ssm_layer(4, 16, 16, 2, conv=4, norm_groups=2, mlp=oracle.dense(48)),
+        oracle.att_layer(4, 2, 16, 8, 0.25, window=36, pool=12, rot_dims=8,
+                         mlp=oracle.routed(6, 2, 16, count=2, keep=1, shared=16))])
+    W = oracle.random_weights(cfg, seed=5)
+    toks = tokens(400, 37, 6)
+    want = {"a": oracle.forward(cfg, oracle.as_f64(W), toks)[0]}
+    eng = engine(write_model(tmp_path, cfg, W), dtype="float32", max_tokens=416, device="cuda")
+    assert eng.runner.graphs
+    check(replay(eng, {"a": toks}, [[("a", 250)]] + [[("a", 1)]] * 150), want, "float32")
+
+
+def test_large_prompt_takes_the_sorted_expert_path(tmp_path):
+    """A prompt portion over the small-batch threshold of the routed feed-forward."""
+    from aws_k8s_ansible_provisioner_amd.models import mudepel
+
+    cfg = oracle.make_config(width=32, vocab=37, layers=[
+        oracle.att_layer(2, 1, 8, 8, 0.4, window=30, pool=10, rot_dims=4,
+                         mlp=oracle.routed(5, 2, 16, shared=8))])
+    W = oracle.random_weights(cfg, seed=6)
+    toks = tokens(mudepel.MOE_DENSE_ROWS + 70, 37, 7)
+    want = {"a": oracle.forward(cfg, oracle.as_f64(W), toks)[0]}
+    eng = engine(write_model(tmp_path, cfg, W), dtype="float32", max_tokens=512, device="cuda")
+    n = mudepel.MOE_DENSE_ROWS + 40
+    check(replay(eng, {"a": toks}, [[("a", n)], [("a", 30)]]), want, "float32")
+
+
+def test_greedy_generation(model):
+    from aws_k8s_ansible_provisioner_amd.engine.config import EngineConfig, SamplingParams
+    from aws_k8s_ansible_provisioner_amd.engine.llm_engine import LLMEngine
+
+    cfg, W, path, _, _ = model
+    eng = LLMEngine(EngineConfig(model=path, load_format="safetensors", weights_path=path,
+                                 dtype="float32", max_model_len=128, max_num_seqs=4,
+                                 max_num_batched_tokens=24, num_gpu_blocks=16, device="cuda",
+                                 gc_freeze=False), log=lambda *a: None)
+    assert eng.runner.graphs
+    prompts = [tokens(n, cfg["vocab"], 20 + n) for n in (30, 3, 17, 9)]
+    outs = eng.generate(None, SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True),
+                        prompt_ids=prompts)
+    assert [len(o.output_ids) for o in outs] == [12] * 4
+    W64 = oracle.as_f64(W)
+    for p, o in zip(prompts, outs):
+        logits = oracle.forward(cfg, W64, p + o.output_ids)[0]
+        for i, tok in enumerate(o.output_ids):
+            row = logits[len(p) - 1 + i]
+            assert row[tok] >= row.max() - 1e-3 * row.std(), (i, tok, int(row.argmax()))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(OTHER))
+def test_other_configurations(tmp_path, name, dtype):
+    cfg = oracle.make_config(**dict({"vocab": 31}, **OTHER[name]))
+    W = oracle.random_weights(cfg, seed=len(name))
+    reqs = {"p": tokens(45, cfg["vocab"], 11), "q": tokens(38, cfg["vocab"], 12)}
+    W64 = oracle.as_f64(W)
+    want = {n: oracle.forward(cfg, W64, t)[0] for n, t in reqs.items()}
+    eng = engine(write_model(tmp_path, cfg, W), dtype=dtype, device="cuda")
+    sched = [[("p", 17), ("q", 2)], [("p", 1), ("q", 30)], [("p", 27), ("q", 1)],
+             [("q", 1)], [("q", 4)]]
+    check(replay(eng, reqs, sched), want, dtype)
+
+
+def test_registry_model_generates_with_sampling():
+    from aws_k8s_ansible_provisioner_amd.engine.config import EngineConfig, SamplingParams
+    from aws_k8s_ansible_provisioner_amd.engine.llm_engine import LLMEngine
+
+    eng = LLMEngine(EngineConfig(model="tiny-mudepel", dtype="bfloat16", max_model_len=256,
+                                 max_num_seqs=4, max_num_batched_tokens=64, num_gpu_blocks=32,
+                                 device="cuda", gc_freeze=False), log=lambda *a: None)
+    outs = eng.generate(None, SamplingParams(max_tokens=20, temperature=0.8, top_p=0.9, seed=3,
+                                             ignore_eos=True),
+                        prompt_ids=[[5, 6, 7], [9] * 70, [1, 2], [3] * 33, [4] * 5])
+    assert [len(o.output_ids) for o in outs] == [20] * 5
+
+
+def test_large_batches_take_the_grouped_expert_gemms():
+    """With the core library loaded, prompt-sized batches of a routed layer run the framework's
+    grouped expert GEMMs (no host round trip); same result as the oracle's experts."""
+    from aws_k8s_ansible_provisioner_amd import ops
+    from aws_k8s_ansible_provisioner_amd.models.config import mudepel_config
+    from aws_k8s_ansible_provisioner_amd.models.mudepel import MudepelLM
+
+    ops.load_native(required=True)
+    cfg = oracle.make_config(width=128, vocab=37, layers=[
+        oracle.ssm_layer(2, 16, 16, 1, mlp=oracle.routed(6, 2, 64, count=3, keep=2, shared=64))])
+    W = oracle.random_weights(cfg, seed=3)
+    m = MudepelLM(mudepel_config("g", cfg), "cuda", dtype=torch.bfloat16, max_model_len=64)
+    m.load_state_dict(W)
+    h = torch.randn(300, 128, generator=gen(5)).bfloat16()
+    assert m._grouped_ok(h.cuda(), 64)
+    want = oracle.moe(h.double(), oracle.as_f64(W), "l0.", cfg["layers"][0]["mlp"])
+    for small in (False, True):
+        ya, yb = m._feed_forward(m.layers[0], h.cuda(), small)
+        got = sum(t.double().cpu() for t in (ya, yb) if t is not None)
+        torch.testing.assert_close(got, want, rtol=3e-2, atol=3e-2)
