@@ -386,19 +386,23 @@ struct ScanArgs {
 
 constexpr int kScanTokens = 16;
 
-// One workgroup per (sequence, head).  Thread (v, part) owns column v of the state rows
-// part, part + NP, ... (NP = 256 / V parts), R of them, in registers over all rows of the step.
-// Tokens are staged 16 at a time (x, B, C, step size and decay); per token a thread updates its
-// rows and adds its share of S^T C; the parts' shares meet in LDS after the 16 tokens.
+__host__ __device__ __forceinline__ int up4(int n) { return (n + 3) & ~3; }
+
+// One workgroup per (sequence, head).  Thread (v, part) owns column v of the R consecutive
+// state rows part R .. part R + R - 1 (NP = 256 / V parts), in registers over all rows of the
+// step.  Tokens are staged TK at a time (x, B, C, step size and decay; TK = 16 for prompt
+// chunks, 1 for steps of single rows); per token a thread updates its rows and adds its share
+// of S^T C, reading B and C from LDS four rows at a time (all lanes of a wave read the same
+// addresses); the parts' shares meet in LDS after the staged tokens.
 template <typename TY, int R>
-__global__ __launch_bounds__(256) void selective_scan_kernel(const ScanArgs a) {
-  extern __shared__ float lds[];
+__global__ __launch_bounds__(256) void selective_scan_kernel(const ScanArgs a, const int TK) {
+  extern __shared__ __align__(16) float lds[];
   const int V = a.V, N = a.N, NP = 256 / V;
-  float* xs = lds;                              // [16][V]
-  float* bs = xs + kScanTokens * V;             // [16][N]
-  float* cs = bs + kScanTokens * N;             // [16][N]
-  float* dts = cs + kScanTokens * N;            // [16] step, [16] decay
-  float* ys = dts + 2 * kScanTokens;            // [16][NP][V]
+  float* xs = lds;                              // [TK][V]
+  float* bs = xs + up4(TK * V);                 // [TK][N]
+  float* cs = bs + up4(TK * N);                 // [TK][N]
+  float* dts = cs + up4(TK * N);                // [TK] step, [TK] decay
+  float* ys = dts + up4(2 * TK);                // [TK][NP][V]
   const int b = blockIdx.x, h = blockIdx.y;
   const int r0 = a.q_start ? a.q_start[b] : b;
   const int r1 = a.q_start ? a.q_start[b + 1] : b + 1;
@@ -409,19 +413,19 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(const ScanArgs a) {
   const int inner = a.H * V, C = inner + 2 * a.G * N;
   const int tid = threadIdx.x;
   const int v = tid % V, part = tid / V;
-  const bool active = part < NP;
+  const int n0 = part * R;
+  const bool active = part < NP && n0 < N;
+  const bool vec = (N & 3) == 0 && (R & 3) == 0;
   float* sp = a.state + ((size_t)slot * a.H + h) * N * V;
   float S[R];
   const bool carry = a.positions[r0] > 0;
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int n = part + r * NP;
-    S[r] = (carry && active && n < N) ? sp[(size_t)n * V + v] : 0.f;
-  }
+  for (int r = 0; r < R; ++r)
+    S[r] = (carry && active && n0 + r < N) ? sp[(size_t)(n0 + r) * V + v] : 0.f;
   const float ea = expf(a.a_log[h]), dsk = a.d_skip[h], dtb = a.dt_bias[h];
   const TY* proj = (const TY*)a.proj;
-  for (int c0 = r0; c0 < r1; c0 += kScanTokens) {
-    const int nt = min(kScanTokens, r1 - c0);
+  for (int c0 = r0; c0 < r1; c0 += TK) {
+    const int nt = min(TK, r1 - c0);
     __syncthreads();
     for (int i = tid; i < nt * V; i += 256) {
       const int tk = i / V, e = i - tk * V;
@@ -437,26 +441,41 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(const ScanArgs a) {
       const float z = ldf(proj + (size_t)(c0 + tid) * a.proj_stride + a.dt_off + h) + dtb;
       const float dt = z > 20.f ? z : log1pf(expf(z));
       dts[tid] = dt;
-      dts[kScanTokens + tid] = expf(-ea * dt);
+      dts[TK + tid] = expf(-ea * dt);
     }
     __syncthreads();
     if (active) {
       for (int tk = 0; tk < nt; ++tk) {
-        const float dt = dts[tk], dec = dts[kScanTokens + tk];
+        const float dt = dts[tk], dec = dts[TK + tk];
         const float dx = dt * xs[tk * V + v];
-        const float* bt = bs + tk * N + part;
-        const float* ct = cs + tk * N + part;
+        const float* bt = bs + tk * N + n0;
+        const float* ct = cs + tk * N + n0;
         float acc = 0.f;
+        if (vec) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-          const int n = r * NP;
-          if (part + n < N) {
-            S[r] = dec * S[r] + dx * bt[n];
-            acc += S[r] * ct[n];
+          for (int r = 0; r < R; r += 4) {
+            if (n0 + r < N) {
+              const float4 b4 = *(const float4*)(bt + r), c4 = *(const float4*)(ct + r);
+              S[r] = dec * S[r] + dx * b4.x;
+              S[r + 1] = dec * S[r + 1] + dx * b4.y;
+              S[r + 2] = dec * S[r + 2] + dx * b4.z;
+              S[r + 3] = dec * S[r + 3] + dx * b4.w;
+              acc += S[r] * c4.x + S[r + 1] * c4.y + S[r + 2] * c4.z + S[r + 3] * c4.w;
+            }
+          }
+        } else {
+#pragma unroll
+          for (int r = 0; r < R; ++r) {
+            if (n0 + r < N) {
+              S[r] = dec * S[r] + dx * bt[r];
+              acc += S[r] * ct[r];
+            }
           }
         }
         ys[(tk * NP + part) * V + v] = acc;
       }
+    } else if (part < NP) {
+      for (int tk = 0; tk < nt; ++tk) ys[(tk * NP + part) * V + v] = 0.f;
     }
     __syncthreads();
     for (int i = tid; i < nt * V; i += 256) {
@@ -468,10 +487,8 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(const ScanArgs a) {
   }
   if (active) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int n = part + r * NP;
-      if (n < N) sp[(size_t)n * V + v] = S[r];
-    }
+    for (int r = 0; r < R; ++r)
+      if (n0 + r < N) sp[(size_t)(n0 + r) * V + v] = S[r];
   }
 }
 
@@ -563,15 +580,18 @@ void launch_selective_scan(float* y, const float* xbc, const void* proj, int pro
   ScanArgs a{y, xbc, proj, dt_bias, a_log, d_skip, state, seq_slot, positions, q_start,
              proj_stride, dt_off, H, V, N, G, T, B};
   const int NP = 256 / V, R = selective_scan_rows(V, N);
-  const size_t lds = (size_t)(kScanTokens * (V + 2 * N + 2 + NP * V)) * sizeof(float);
+  const int TK = q_start ? kScanTokens : 1;
+  const size_t lds = (size_t)(up4(TK * V) + 2 * up4(TK * N) + up4(2 * TK) + TK * NP * V) *
+                     sizeof(float);
   const dim3 grid(B, H);
-#define AKAP_SCAN(TY, RR) selective_scan_kernel<TY, RR><<<grid, 256, lds, s>>>(a)
-#define AKAP_SCAN_R(TY)               \
-  do {                                \
-    if (R <= 8) AKAP_SCAN(TY, 8);     \
+#define AKAP_SCAN(TY, RR) selective_scan_kernel<TY, RR><<<grid, 256, lds, s>>>(a, TK)
+#define AKAP_SCAN_R(TY)                  \
+  do {                                   \
+    if (R <= 4) AKAP_SCAN(TY, 4);        \
+    else if (R <= 8) AKAP_SCAN(TY, 8);   \
     else if (R <= 16) AKAP_SCAN(TY, 16); \
     else if (R <= 32) AKAP_SCAN(TY, 32); \
-    else AKAP_SCAN(TY, 64);           \
+    else AKAP_SCAN(TY, 64);              \
   } while (0)
   if (f32) AKAP_SCAN_R(float);
   else AKAP_SCAN_R(bf16);

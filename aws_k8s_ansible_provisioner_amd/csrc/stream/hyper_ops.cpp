@@ -200,10 +200,10 @@ void bias_rope_cache(Tensor proj, Tensor q_out, Tensor k_cache, Tensor v_cache, 
                   slots.numel() >= T, "bias_rope_cache: shapes");
   TORCH_CHECK(q_off >= 0 && q_off + H * D <= N && k_off >= 0 && k_off + G * D <= N && v_off >= 0 &&
                   v_off + G * Dv <= N, "bias_rope_cache: column ranges");
-  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.size(1) == G &&
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 5 && k_cache.size(1) == G &&
                   k_cache.size(3) == D && v_cache.size(0) == k_cache.size(0) &&
-                  v_cache.size(1) == G && v_cache.size(2) == k_cache.size(2) &&
-                  v_cache.size(3) == Dv, "bias_rope_cache: cache shapes");
+                  v_cache.size(1) == G && v_cache.size(2) * 8 == k_cache.size(2) &&
+                  v_cache.size(3) == Dv && v_cache.size(4) == 8, "bias_rope_cache: cache shapes");
   const bool f32 = is_f32(proj, "proj");
   TORCH_CHECK(q_out.scalar_type() == proj.scalar_type() &&
                   k_cache.scalar_type() == proj.scalar_type() &&
@@ -232,9 +232,9 @@ void check_paged(const Tensor& k_cache, const Tensor& v_cache, const std::option
                  int64_t* PS) {
   CHECK_GPU(k_cache); CHECK_GPU(v_cache); CHECK_CONTIG(k_cache); CHECK_CONTIG(v_cache);
   CHECK_GPU(block_tables); CHECK_I32(block_tables); CHECK_CONTIG(block_tables);
-  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && block_tables.dim() == 2 &&
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 5 && block_tables.dim() == 2 &&
                   v_cache.size(0) == k_cache.size(0) && v_cache.size(1) == k_cache.size(1) &&
-                  v_cache.size(2) == k_cache.size(2) &&
+                  v_cache.size(2) * 8 == k_cache.size(2) && v_cache.size(4) == 8 &&
                   v_cache.scalar_type() == k_cache.scalar_type(), "paged cache shapes");
   *PS = 0;
   if (pool > 0) {
@@ -282,11 +282,12 @@ void pool_cache_blocks(Tensor k_cache, Tensor v_cache, Tensor k_pool, Tensor v_p
   akap_stream::launch_pool_cache_blocks(p, is_f32(k_cache, "k_cache"), cur_stream());
 }
 
-void pooled_window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
-                             std::optional<Tensor> k_pool, std::optional<Tensor> v_pool,
-                             Tensor block_tables, std::optional<Tensor> q_start, Tensor positions,
-                             Tensor slots, double scale, int64_t window, int64_t pool,
-                             bool unit_sink) {
+akap_stream::PoolAttnParams attn_params(Tensor& out, Tensor& q, Tensor& k_cache, Tensor& v_cache,
+                                        std::optional<Tensor>& k_pool,
+                                        std::optional<Tensor>& v_pool, Tensor& block_tables,
+                                        std::optional<Tensor>& q_start, Tensor& positions,
+                                        Tensor& slots, double scale, int64_t window, int64_t pool,
+                                        bool unit_sink) {
   int64_t PS;
   if (window <= 0) pool = 0;
   check_paged(k_cache, v_cache, k_pool, v_pool, block_tables, pool, &PS);
@@ -296,6 +297,7 @@ void pooled_window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cach
   TORCH_CHECK(q.dim() == 3 && out.dim() == 2 && out.size(0) == q.size(0), "attention: shapes");
   const int64_t T = q.size(0), H = q.size(1), D = q.size(2);
   const int64_t G = k_cache.size(1), Dv = v_cache.size(3);
+  TORCH_CHECK(k_cache.size(2) % 8 == 0, "attention: the block size must be a multiple of 8");
   TORCH_CHECK(k_cache.size(3) == D && H % G == 0 && H / G <= 16 && Dv <= 256 && D <= 512 &&
                   out.size(1) >= H * Dv, "attention: head sizes (at most 16 query heads per "
               "key/value head, values of at most 256 entries)");
@@ -319,8 +321,65 @@ void pooled_window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cach
   TORCH_CHECK(p.B >= 1 && p.B <= block_tables.size(0), "attention: a block-table row per sequence");
   p.H = (int)H; p.G = (int)G; p.D = (int)D; p.Dv = (int)Dv; p.BS = (int)k_cache.size(2);
   p.PS = (int)PS; p.window = (int)window; p.pool = (int)pool; p.unit_sink = unit_sink ? 1 : 0;
+  return p;
+}
+
+void pooled_window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
+                             std::optional<Tensor> k_pool, std::optional<Tensor> v_pool,
+                             Tensor block_tables, std::optional<Tensor> q_start, Tensor positions,
+                             Tensor slots, double scale, int64_t window, int64_t pool,
+                             bool unit_sink) {
+  const akap_stream::PoolAttnParams p =
+      attn_params(out, q, k_cache, v_cache, k_pool, v_pool, block_tables, q_start, positions,
+                  slots, scale, window, pool, unit_sink);
   const c10::DeviceGuard g(q.device());
   akap_stream::launch_pooled_window_attention(p, is_f32(q, "q"), cur_stream());
+}
+
+void pooled_window_attention_decode_mfma(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
+                                         std::optional<Tensor> k_pool,
+                                         std::optional<Tensor> v_pool, Tensor block_tables,
+                                         Tensor positions, Tensor slots, double scale,
+                                         int64_t window, int64_t pool, bool unit_sink) {
+  std::optional<Tensor> none;
+  const akap_stream::PoolAttnParams p =
+      attn_params(out, q, k_cache, v_cache, k_pool, v_pool, block_tables, none, positions, slots,
+                  scale, window, pool, unit_sink);
+  TORCH_CHECK(q.scalar_type() == at::kBFloat16, "matrix-core attention: bf16 only");
+  TORCH_CHECK(akap_stream::pooled_mfma_supported(p.H, p.G, p.D, p.Dv, p.BS) && p.H / p.G <= 32,
+              "matrix-core attention: unsupported head sizes");
+  const c10::DeviceGuard g(q.device());
+  akap_stream::launch_pooled_window_decode_mfma(p, p.T, cur_stream());
+}
+
+bool pooled_mfma_supported(int64_t H, int64_t G, int64_t D, int64_t Dv, int64_t BS) {
+  return akap_stream::pooled_mfma_supported((int)H, (int)G, (int)D, (int)Dv, (int)BS);
+}
+
+void pooled_window_attention_prefill_mfma(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
+                                          std::optional<Tensor> k_pool,
+                                          std::optional<Tensor> v_pool, Tensor block_tables,
+                                          Tensor q_start, Tensor positions, Tensor slots,
+                                          Tensor tile_seq, Tensor tile_row, int64_t tile_rows,
+                                          double scale, int64_t window, int64_t pool,
+                                          bool unit_sink) {
+  std::optional<Tensor> qs(q_start);
+  const akap_stream::PoolAttnParams p =
+      attn_params(out, q, k_cache, v_cache, k_pool, v_pool, block_tables, qs, positions, slots,
+                  scale, window, pool, unit_sink);
+  TORCH_CHECK(q.scalar_type() == at::kBFloat16, "matrix-core attention: bf16 only");
+  TORCH_CHECK(akap_stream::pooled_mfma_supported(p.H, p.G, p.D, p.Dv, p.BS),
+              "matrix-core attention: unsupported head sizes");
+  TORCH_CHECK(tile_rows == 128, "matrix-core attention: tiles of 128 rows");
+  TORCH_CHECK(out.stride(0) % 4 == 0 && (uintptr_t)out.data_ptr() % 8 == 0,
+              "matrix-core attention: out rows must start at multiples of 8 bytes");
+  CHECK_GPU(tile_seq); CHECK_GPU(tile_row); CHECK_I32(tile_seq); CHECK_I32(tile_row);
+  CHECK_CONTIG(tile_seq); CHECK_CONTIG(tile_row);
+  TORCH_CHECK(tile_seq.numel() == tile_row.numel(), "matrix-core attention: tile map");
+  const c10::DeviceGuard g(q.device());
+  akap_stream::launch_pooled_window_prefill_mfma(p, tile_seq.data_ptr<int32_t>(),
+                                                 tile_row.data_ptr<int32_t>(),
+                                                 (int)tile_seq.numel(), cur_stream());
 }
 
 }  // namespace
@@ -347,6 +406,15 @@ TORCH_LIBRARY_FRAGMENT(akap_stream, m) {
   m.def("pooled_window_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, "
         "Tensor? k_pool, Tensor? v_pool, Tensor block_tables, Tensor? q_start, Tensor positions, "
         "Tensor slots, float scale, int window, int pool, bool unit_sink) -> ()");
+  m.def("pooled_window_attention_decode_mfma(Tensor(a!) out, Tensor q, Tensor k_cache, "
+        "Tensor v_cache, Tensor? k_pool, Tensor? v_pool, Tensor block_tables, Tensor positions, "
+        "Tensor slots, float scale, int window, int pool, bool unit_sink) -> ()");
+  m.def("pooled_mfma_supported(int H, int G, int D, int Dv, int BS) -> bool",
+        &pooled_mfma_supported);
+  m.def("pooled_window_attention_prefill_mfma(Tensor(a!) out, Tensor q, Tensor k_cache, "
+        "Tensor v_cache, Tensor? k_pool, Tensor? v_pool, Tensor block_tables, Tensor q_start, "
+        "Tensor positions, Tensor slots, Tensor tile_seq, Tensor tile_row, int tile_rows, "
+        "float scale, int window, int pool, bool unit_sink) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(akap_stream, CUDA, m) {
@@ -359,4 +427,6 @@ TORCH_LIBRARY_IMPL(akap_stream, CUDA, m) {
   m.impl("bias_rope_cache", &bias_rope_cache);
   m.impl("pool_cache_blocks", &pool_cache_blocks);
   m.impl("pooled_window_attention", &pooled_window_attention);
+  m.impl("pooled_window_attention_prefill_mfma", &pooled_window_attention_prefill_mfma);
+  m.impl("pooled_window_attention_decode_mfma", &pooled_window_attention_decode_mfma);
 }

@@ -7,8 +7,9 @@
 //   pooled_window_attention  one online softmax over pooled entries and window tokens, optionally
 //                          starting from a sink of score 0 (a 1 in the denominator)
 //
-// K [NB, G, BS, D], V [NB, G, BS, Dv] token-major in the activation type; pooled K / V
-// [NB, G, PS, D / Dv] fp32.  Biases, angles, scores, softmax and the weighted sums are fp32.
+// K [NB, G, BS, D] token-major and V [NB, G, BS / 8, Dv, 8] (groups of 8 tokens,
+// dimension-major inside a group: the layout the matrix-core kernels read) in the activation
+// type; pooled K / V [NB, G, PS, D / Dv] fp32.  Biases, angles, scores, softmax and the weighted sums are fp32.
 #include "../kernels/common.h"
 #include "stream.h"
 
@@ -103,7 +104,8 @@ __global__ __launch_bounds__(256) void bias_rope_cache_kernel(const RopeCachePar
       if (e < nq + nk)
         stf((T*)p.k_cache + ((blk * p.G + head) * p.BS + off) * p.D + i, val);
       else
-        stf((T*)p.v_cache + ((blk * p.G + head) * p.BS + off) * p.Dv + i, val);
+        stf((T*)p.v_cache + (((blk * p.G + head) * (p.BS >> 3) + (off >> 3)) * p.Dv + i) * 8 +
+                (off & 7), val);
     }
   }
 }
@@ -113,25 +115,38 @@ __global__ __launch_bounds__(256) void bias_rope_cache_kernel(const RopeCachePar
 template <typename T>
 __global__ __launch_bounds__(128) void pool_cache_blocks_kernel(const PoolParams p) {
   const int t = blockIdx.x, g = blockIdx.y;
-  const int64_t pos = p.positions[t];
+  const int pos = (int)p.positions[t];
   if (p.slots[t] < 0 || (pos + 1) % p.pool) return;
   const int b = p.q_start ? seq_of_row(p.q_start, p.B, t) : t;
   const int32_t* bt = p.block_tables + (size_t)b * p.max_blocks;
-  const int64_t first = pos + 1 - p.pool;
-  const int64_t page0 = bt[first / p.BS];
-  const int idx = (int)((first % p.BS) / p.pool);
+  const int first = pos + 1 - p.pool;
+  const int page0 = bt[first / p.BS];
+  const int idx = (first % p.BS) / p.pool;
   const float inv = 1.0f / (float)p.pool;
+  const T* kc = (const T*)p.k_cache;
+  const T* vc = (const T*)p.v_cache;
   for (int i = threadIdx.x; i < p.D + p.Dv; i += 128) {
     const bool isk = i < p.D;
-    const int e = isk ? i : i - p.D, n = isk ? p.D : p.Dv;
-    const T* base = (const T*)(isk ? p.k_cache : p.v_cache);
+    const int e = isk ? i : i - p.D;
     float acc = 0.f;
-    for (int j = 0; j < p.pool; ++j) {
-      const int64_t q = first + j, page = bt[q / p.BS], off = q % p.BS;
-      acc += ldf(base + ((page * p.G + g) * p.BS + off) * n + e);
+    int q = first;
+    while (q <= pos) {                       // page by page
+      const int page = bt[q / p.BS], off0 = q % p.BS;
+      const int cnt = min(pos + 1 - q, p.BS - off0);
+      const size_t row = (size_t)page * p.G + g;
+      if (isk) {
+        const T* src = kc + (row * p.BS + off0) * p.D + e;
+        for (int j = 0; j < cnt; ++j) acc += ldf(src + (size_t)j * p.D);
+      } else {
+        for (int j = 0; j < cnt; ++j) {
+          const int off = off0 + j;
+          acc += ldf(vc + ((row * (p.BS >> 3) + (off >> 3)) * p.Dv + e) * 8 + (off & 7));
+        }
+      }
+      q += cnt;
     }
-    float* dst = isk ? p.k_pool : p.v_pool;
-    dst[((page0 * p.G + g) * p.PS + idx) * n + e] = acc * inv;
+    if (isk) p.k_pool[(((size_t)page0 * p.G + g) * p.PS + idx) * p.D + e] = acc * inv;
+    else p.v_pool[(((size_t)page0 * p.G + g) * p.PS + idx) * p.Dv + e] = acc * inv;
   }
 }
 
@@ -152,11 +167,11 @@ __global__ void pooled_window_attention_kernel(const PoolAttnParams p) {
   if (p.slots[t] < 0) return;
   const int b = p.q_start ? seq_of_row(p.q_start, p.B, t) : t;
   const int32_t* bt = p.block_tables + (size_t)b * p.max_blocks;
-  const int64_t i = p.positions[t];
-  const int64_t lo = p.window > 0 ? (i - p.window + 1 > 0 ? i - p.window + 1 : 0) : 0;
-  const int64_t nb = (p.pool > 0 && p.window > 0 && i - p.window + 1 > 0)
-                         ? (i - p.window + 1) / p.pool : 0;
-  const int64_t n = nb + (i - lo + 1);
+  const int i = (int)p.positions[t];
+  const int lo = p.window > 0 ? (i - p.window + 1 > 0 ? i - p.window + 1 : 0) : 0;
+  const int nb = (p.pool > 0 && p.window > 0 && i - p.window + 1 > 0)
+                     ? (i - p.window + 1) / p.pool : 0;
+  const int n = nb + (i - lo + 1);
   float* qs = lds + (size_t)wave * (p.D + 64);
   float* ps = qs + p.D;
   const T* q = (const T*)p.q + ((size_t)t * p.H + h) * p.D;
@@ -169,17 +184,17 @@ __global__ void pooled_window_attention_kernel(const PoolAttnParams p) {
   for (int k = 0; k < kMaxDv / 64; ++k) acc[k] = 0.f;
   const T* kc = (const T*)p.k_cache;
   const T* vc = (const T*)p.v_cache;
-  for (int64_t base = 0; base < n; base += 64) {
-    const int64_t idx = base + lane;
+  for (int base = 0; base < n; base += 64) {
+    const int idx = base + lane;
     float s = -INFINITY;
     if (idx < n) {
       if (idx < nb) {
-        const int64_t first = idx * p.pool, page = bt[first / p.BS];
-        const int e = (int)((first % p.BS) / p.pool);
-        s = dot_row(qs, p.k_pool + ((page * p.G + g) * p.PS + e) * p.D, p.D);
+        const int first = idx * p.pool, page = bt[first / p.BS];
+        const int e = (first % p.BS) / p.pool;
+        s = dot_row(qs, p.k_pool + (((size_t)page * p.G + g) * p.PS + e) * p.D, p.D);
       } else {
-        const int64_t j = lo + (idx - nb), page = bt[j / p.BS], off = j % p.BS;
-        s = dot_row(qs, kc + ((page * p.G + g) * p.BS + off) * p.D, p.D);
+        const int j = lo + (idx - nb), page = bt[j / p.BS], off = j % p.BS;
+        s = dot_row(qs, kc + (((size_t)page * p.G + g) * p.BS + off) * p.D, p.D);
       }
     }
     const float mx = fmaxf(m, wave_max(s));
@@ -191,23 +206,24 @@ __global__ void pooled_window_attention_kernel(const PoolAttnParams p) {
     m = mx;
     ps[lane] = w;
     __syncthreads();
-    const int cnt = (int)(n - base < 64 ? n - base : 64);
+    const int cnt = n - base < 64 ? n - base : 64;
     for (int kk = 0; kk < cnt; ++kk) {
-      const int64_t id2 = base + kk;
+      const int id2 = base + kk;
       const float w2 = ps[kk];
       if (id2 < nb) {
-        const int64_t first = id2 * p.pool, page = bt[first / p.BS];
-        const int e = (int)((first % p.BS) / p.pool);
-        const float* vr = p.v_pool + ((page * p.G + g) * p.PS + e) * p.Dv;
+        const int first = id2 * p.pool, page = bt[first / p.BS];
+        const int e = (first % p.BS) / p.pool;
+        const float* vr = p.v_pool + (((size_t)page * p.G + g) * p.PS + e) * p.Dv;
 #pragma unroll
         for (int k = 0; k < kMaxDv / 64; ++k)
           if (lane + 64 * k < p.Dv) acc[k] += w2 * vr[lane + 64 * k];
       } else {
-        const int64_t j = lo + (id2 - nb), page = bt[j / p.BS], off = j % p.BS;
-        const T* vr = vc + ((page * p.G + g) * p.BS + off) * p.Dv;
+        const int j = lo + (id2 - nb), page = bt[j / p.BS], off = j % p.BS;
+        const T* vr = vc + (((size_t)page * p.G + g) * (p.BS >> 3) + (off >> 3)) * p.Dv * 8 +
+                      (off & 7);
 #pragma unroll
         for (int k = 0; k < kMaxDv / 64; ++k)
-          if (lane + 64 * k < p.Dv) acc[k] += w2 * ldf(vr + lane + 64 * k);
+          if (lane + 64 * k < p.Dv) acc[k] += w2 * ldf(vr + (size_t)(lane + 64 * k) * 8);
       }
     }
     __syncthreads();

@@ -292,7 +292,7 @@ struct RopeCacheParams {
   int proj_stride;
   void* q_out;           // [T, H, D]
   void* k_cache;         // [NB, G, BS, D]
-  void* v_cache;         // [NB, G, BS, Dv]
+  void* v_cache;         // [NB, G, BS / 8, Dv, 8]
   const int64_t* positions;
   const int64_t* slots;
   const float* cos_sin;  // [max_pos, rot_dims] = [cos | sin], or null
@@ -332,5 +332,14 @@ struct PoolAttnParams {
   int max_blocks, T, B, H, G, D, Dv, BS, PS, window, pool, unit_sink;
 };
 void launch_pooled_window_attention(const PoolAttnParams& p, bool f32, hipStream_t s);
+// matrix-core form for prompt chunks (bf16): the rows of the tile map (tile_seq / tile_row:
+// sequence and first chunk row of a tile of 128 tokens)
+bool pooled_mfma_supported(int H, int G, int D, int Dv, int BS);
+void launch_pooled_window_prefill_mfma(const PoolAttnParams& p, const int32_t* tile_seq,
+                                       const int32_t* tile_row, int num_tiles, hipStream_t s);
+// matrix-core form for one query per sequence (row t = sequence t, the first `rows` rows): the
+// query heads of a key/value head are the columns of a tile, the key range is split over the
+// workgroup's waves
+void launch_pooled_window_decode_mfma(const PoolAttnParams& p, int rows, hipStream_t s);
 
 }  // namespace akap_stream

@@ -299,13 +299,17 @@ class MudepelLM:
 
     def allocate_kv_segments(self, num_blocks: int, block_size: int, kv_dtype: str = "auto",
                              max_segment_bytes: Optional[int] = None) -> list:
-        """Per layer run with an attention: K [NB, G, BS, D] and V [NB, G, BS, Dv] (token-major
-        rows) in the model's dtype, and for a pooled mask the fp32 entries K [NB, G, n, D],
+        """Per layer run with an attention: K [NB, G, BS, D] (token-major rows) and V
+        [NB, G, BS / 8, Dv, 8] (groups of 8 tokens, dimension-major inside a group: what a
+        matrix-core operand contracts over is one 16-byte load) in the model's dtype, and for a
+        pooled mask the fp32 entries K [NB, G, n, D],
         V [NB, G, n, Dv] of the blocks that start in each page (n = ceil(BS / pool)), kept by
         the model beside the pages they belong to.  State-space layers cache nothing per
         token."""
         if kv_dtype not in ("auto", "bf16", "bfloat16"):
             raise ValueError("Mudepel: the KV cache is kept in the model's dtype (no fp8)")
+        if block_size % 8:
+            raise ValueError("Mudepel: the block size must be a multiple of 8")
         segs, self._seg_map, self.pooled = [], {}, {}
         for r, i in enumerate(self.runs):
             m = self.cfg.layer_specs[i].mixer
@@ -314,8 +318,8 @@ class MudepelLM:
             self._seg_map[r] = len(segs)
             segs.append(torch.zeros(num_blocks, m.kv_heads, block_size, m.dim, dtype=self.dtype,
                                     device=self.device))
-            segs.append(torch.zeros(num_blocks, m.kv_heads, block_size, m.vdim, dtype=self.dtype,
-                                    device=self.device))
+            segs.append(torch.zeros(num_blocks, m.kv_heads, block_size // 8, m.vdim, 8,
+                                    dtype=self.dtype, device=self.device))
             if m.pool > 0:
                 n = sops.pool_slots(block_size, m.pool)
                 self.pooled[r] = (
@@ -383,9 +387,15 @@ class MudepelLM:
             sops.pool_cache_blocks(kc, vc, kp, vp, batch.positions, batch.slots,
                                    batch.block_tables, q_start, m.pool)
         att = torch.empty(T, m.heads * m.vdim, dtype=self.dtype, device=self.device)
-        sops.pooled_window_attention(att, q, kc, vc, kp, vp, batch.block_tables, q_start,
-                                     batch.positions, batch.slots, m.scale, m.window, m.pool,
-                                     m.unit_sink)
+        if batch.is_prefill:
+            sops.pooled_window_attention_prefill(
+                att, q, kc, vc, kp, vp, batch.block_tables, q_start, batch.positions, batch.slots,
+                batch.tile_seq, batch.tile_row, batch.tile_rows, m.scale, m.window, m.pool,
+                m.unit_sink, first_seq=batch.num_decode)
+        else:
+            sops.pooled_window_attention_decode(att, q, kc, vc, kp, vp, batch.block_tables,
+                                                batch.positions, batch.slots, m.scale, m.window,
+                                                m.pool, m.unit_sink)
         return self._linear(att, lw.w_o)
 
     def _state_space(self, lw: StreamLayerWeights, m: StateSpaceSpec, h, batch: AttnBatch,

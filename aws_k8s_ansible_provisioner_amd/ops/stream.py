@@ -1030,8 +1030,8 @@ def bias_rope_cache(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tens
     bias (fp32 [N], laid out like proj's columns; None: no biases); q and k are rotated per head
     on their first cos_sin.shape[1] dimensions in the rotate-half layout (entry i with
     i + dims/2) by the table row of positions[t] (fp32).  q goes to q_out [T, H, D]; k to
-    k_cache [NB, G, BS, D] and v to v_cache [NB, G, BS, Dv] (token-major) at slots[t]; slot -1
-    writes nothing."""
+    k_cache [NB, G, BS, D] and v to v_cache [NB, G, BS / 8, Dv, 8] at slots[t]; slot -1 writes
+    nothing."""
     if _native(proj):
         torch.ops.akap_stream.bias_rope_cache(proj, q_out, k_cache, v_cache, positions, slots,
                                               cos_sin, bias, H, G, D, Dv, q_off, k_off, v_off)
@@ -1050,7 +1050,7 @@ def bias_rope_cache(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tens
     ok = slots >= 0
     sl = slots[ok].long()
     k_cache[sl // BS, :, sl % BS] = k[ok].to(k_cache.dtype)
-    v_cache[sl // BS, :, sl % BS] = v[ok].to(v_cache.dtype)
+    v_cache[sl // BS, :, (sl % BS) // 8, :, sl % 8] = v[ok].to(v_cache.dtype)
 
 
 def _row_sequences(T: int, q_start: Optional[torch.Tensor]):
@@ -1085,7 +1085,7 @@ def pool_cache_blocks(k_cache: torch.Tensor, v_cache: torch.Tensor, k_pool: torc
             pos = torch.arange(first, p + 1)
             pages = block_tables[b][pos // BS].long()
             kk = k_cache[pages, :, pos % BS].float().mean(dim=0)
-            vv = v_cache[pages, :, pos % BS].float().mean(dim=0)
+            vv = v_cache[pages, :, (pos % BS) // 8, :, pos % 8].float().mean(dim=0)
             page, idx = int(block_tables[b][first // BS]), (first % BS) // pool
             k_pool[page, :, idx] = kk
             v_pool[page, :, idx] = vv
@@ -1096,14 +1096,15 @@ def pooled_window_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.T
                             v_pool: Optional[torch.Tensor], block_tables: torch.Tensor,
                             q_start: Optional[torch.Tensor], positions: torch.Tensor,
                             slots: torch.Tensor, scale: float, window: int, pool: int,
-                            unit_sink: bool) -> None:
+                            unit_sink: bool, first_seq: int = 0) -> None:
     """Paged attention of the token rows of a step.  The query at position i of sequence b
     (rows by q_start as in pool_cache_blocks) sees the cached tokens j <= i with i - j < window
     (window 0: all) and, with pool > 0, the pooled entry of every block c with
     c pool + pool - 1 <= i - window (pool_cache_blocks' layout); tokens and blocks share one
     softmax over scale q.k, with 1 added to its denominator when unit_sink.  Query head h reads
     key/value head h // (H / G).  Scores, softmax and the weighted sums are fp32.  Rows with
-    slot -1 are padding and left unwritten.  out [T, >= H Dv]."""
+    slot -1 are padding and left unwritten.  out [T, >= H Dv].  K [NB, G, BS, D] token-major,
+    V [NB, G, BS / 8, Dv, 8].  first_seq (CPU tensors): sequences before it are skipped."""
     if _native(q):
         torch.ops.akap_stream.pooled_window_attention(out, q, k_cache, v_cache, k_pool, v_pool,
                                                       block_tables, q_start, positions, slots,
@@ -1114,6 +1115,8 @@ def pooled_window_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.T
     G, BS, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
     rep = H // G
     for b, (r0, r1) in enumerate(_row_sequences(T, q_start)):
+        if b < first_seq:
+            continue
         for t in range(r0, r1):
             if int(slots[t]) < 0:
                 continue
@@ -1122,7 +1125,7 @@ def pooled_window_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.T
             pos = torch.arange(lo, i + 1)
             pages = block_tables[b][pos // BS].long()
             K = k_cache[pages, :, pos % BS].float()            # [n, G, D]
-            V = v_cache[pages, :, pos % BS].float()
+            V = v_cache[pages, :, (pos % BS) // 8, :, pos % 8].float()
             nb = (i - window + 1) // pool if (pool > 0 and window > 0 and i - window + 1 > 0) \
                 else 0
             if nb > 0:
@@ -1138,6 +1141,62 @@ def pooled_window_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.T
                 e = torch.exp(s - m)
                 den = e.sum() + (torch.exp(-m) if unit_sink else 0.0)
                 out[t, h * Dv:(h + 1) * Dv] = ((e / den) @ V[:, h // rep]).to(out.dtype)
+
+
+def pooled_mfma_ok(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor) -> bool:
+    """Can the matrix-core kernel take these prompt chunks (bf16 on the GPU, head size a
+    multiple of 16, value size 32 / 64 / 128 / 256)?"""
+    if not (q.is_cuda and q.dtype == torch.bfloat16):
+        return False
+    load_native(required=True)
+    return bool(torch.ops.akap_stream.pooled_mfma_supported(
+        q.shape[1], k_cache.shape[1], q.shape[2], v_cache.shape[3], k_cache.shape[2]))
+
+
+def pooled_window_attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
+                                   v_cache: torch.Tensor, k_pool: Optional[torch.Tensor],
+                                   v_pool: Optional[torch.Tensor], block_tables: torch.Tensor,
+                                   positions: torch.Tensor, slots: torch.Tensor, scale: float,
+                                   window: int, pool: int, unit_sink: bool) -> None:
+    """pooled_window_attention for one query per sequence (row t is sequence t).  bf16 rows with
+    matrix-core sizes run on the matrix cores: the query heads of a key/value head are the
+    columns of a tile, so a group reads its keys once, and the key range is split over the
+    waves of a workgroup; everything else on the row kernel."""
+    if pooled_mfma_ok(q, k_cache, v_cache) and q.shape[1] // k_cache.shape[1] <= 32:
+        torch.ops.akap_stream.pooled_window_attention_decode_mfma(
+            out, q, k_cache, v_cache, k_pool, v_pool, block_tables, positions, slots,
+            float(scale), int(window), int(pool), bool(unit_sink))
+        return
+    pooled_window_attention(out, q, k_cache, v_cache, k_pool, v_pool, block_tables, None,
+                            positions, slots, scale, window, pool, unit_sink)
+
+
+def pooled_window_attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
+                                    v_cache: torch.Tensor, k_pool: Optional[torch.Tensor],
+                                    v_pool: Optional[torch.Tensor], block_tables: torch.Tensor,
+                                    q_start: torch.Tensor, positions: torch.Tensor,
+                                    slots: torch.Tensor, tile_seq: torch.Tensor,
+                                    tile_row: torch.Tensor, tile_rows: int, scale: float,
+                                    window: int, pool: int, unit_sink: bool,
+                                    first_seq: int = 0) -> None:
+    """pooled_window_attention for a step with prompt chunks.  The tile map (tile_seq, tile_row:
+    a sequence and the first chunk row of a tile of tile_rows tokens) covers the sequences from
+    first_seq on; the sequences before it are the single rows of a mixed step.  bf16 chunks with
+    matrix-core sizes run on the matrix cores (pooled entries rounded to bf16 operands), the
+    leading single rows and everything else on the row kernel."""
+    if pooled_mfma_ok(q, k_cache, v_cache) and tile_rows == 128 and out.stride(0) % 4 == 0:
+        nd = first_seq
+        if nd:
+            pooled_window_attention_decode(out[:nd], q[:nd], k_cache, v_cache, k_pool, v_pool,
+                                           block_tables, positions[:nd], slots[:nd], scale,
+                                           window, pool, unit_sink)
+        torch.ops.akap_stream.pooled_window_attention_prefill_mfma(
+            out, q, k_cache, v_cache, k_pool, v_pool, block_tables, q_start, positions, slots,
+            tile_seq, tile_row, int(tile_rows), float(scale), int(window), int(pool),
+            bool(unit_sink))
+        return
+    pooled_window_attention(out, q, k_cache, v_cache, k_pool, v_pool, block_tables, q_start,
+                            positions, slots, scale, window, pool, unit_sink)
 
 
 # ----------------------------------------------------------------------------- selective state space

@@ -158,7 +158,7 @@ def test_streams_read_mix_write_and_norm():
     "factor": 8.0, "original": 16, "fast": 2.0, "slow": 0.5})])
 def test_rotation_biases_and_cache_write(dims, scaling):
     g = torch.Generator().manual_seed(dims)
-    T, H, G, D, Dv, BS = 9, 4, 2, 8, 6, 4
+    T, H, G, D, Dv, BS = 9, 4, 2, 8, 6, 8
     rot = {"dims": dims, "base": 50.0, "scaling": scaling}
     N = H * D + G * D + G * Dv + 3
     proj, bias = torch.randn(T, N, generator=g), torch.randn(N, generator=g)
@@ -166,7 +166,7 @@ def test_rotation_biases_and_cache_write(dims, scaling):
     slots = torch.tensor([8, 9, 10, 11, 3, -1, 17, 0, 19])
     cs = sops.rotary_table_yarn(128, dims, 50.0, scaling)
     q = torch.zeros(T, H, D)
-    kc, vc = torch.zeros(5, G, BS, D), torch.zeros(5, G, BS, Dv)
+    kc, vc = torch.zeros(3, G, BS, D), torch.zeros(3, G, BS // 8, Dv, 8)
     sops.bias_rope_cache(proj, q, kc, vc, pos, slots, cs, bias, H, G, D, Dv, 1, 1 + H * D,
                          1 + (H + G) * D)
     p = (proj + bias).to(F64)
@@ -177,7 +177,8 @@ def test_rotation_biases_and_cache_write(dims, scaling):
     for t, s in enumerate(slots.tolist()):
         if s >= 0:
             torch.testing.assert_close(kc[s // BS, :, s % BS].to(F64), wk[t], rtol=1e-5, atol=1e-5)
-            torch.testing.assert_close(vc[s // BS, :, s % BS].to(F64), wv[t], rtol=1e-5, atol=1e-5)
+            torch.testing.assert_close(sops.v_tokens(vc)[s // BS, :, s % BS].to(F64), wv[t],
+                                       rtol=1e-5, atol=1e-5)
     assert kc.abs().sum(dim=(1, 3)).flatten().count_nonzero() == 8     # the padding row wrote nothing
     if scaling is not None:       # scaling changes slow frequencies and the size of cos / sin
         plain = oracle.rotate_half(p[:, 1:1 + H * D].reshape(T, H, D), pos.tolist(),
@@ -195,6 +196,7 @@ def _paged(seed, n, G, D, Dv, BS, pool):
     pos = torch.arange(n)
     slots = perm[pos // BS].long() * BS + pos % BS
     kc[slots // BS, :, slots % BS], vc[slots // BS, :, slots % BS] = k, v
+    vc = sops.v_from_tokens(vc)          # the value cache keeps groups of 8 tokens
     PS = sops.pool_slots(BS, pool)
     kp = torch.full((NB, G, max(1, PS), D), 9.0) if pool else None
     vp = torch.full((NB, G, max(1, PS), Dv), 9.0) if pool else None
@@ -233,7 +235,7 @@ def _attend_want(c, q, first, scale, window):
 
 
 @pytest.mark.parametrize("window,pool,BS,step", [(44, 12, 32, 64), (11, 3, 8, 5), (7, 20, 16, 1),
-                                                 (24, 8, 32, 13), (16, 16, 16, 300), (5, 1, 4, 2)])
+                                                 (24, 8, 32, 13), (16, 16, 16, 300), (5, 1, 8, 2)])
 def test_window_and_pooled_blocks(window, pool, BS, step):
     """Random queries over 150 cached tokens: windows and blocks cut by pages, blocks larger
     than a page and of one token, pooled entries written by steps of several sizes."""

@@ -166,7 +166,7 @@ def _attention_case(dtype, H, G, D, Dv, rot, window, pool, BS, dev, steps, g, si
     NB = 24
     N = H * D + G * (D + Dv) + 3
     kc = torch.zeros(NB, G, BS, D, dtype=dt, device=dev)
-    vc = torch.zeros(NB, G, BS, Dv, dtype=dt, device=dev)
+    vc = torch.zeros(NB, G, BS // 8, Dv, 8, dtype=dt, device=dev)
     PS = sops.pool_slots(BS, pool)
     kp = torch.full((NB, G, max(PS, 1), D), 5.0, device=dev) if pool else None
     vp = torch.full((NB, G, max(PS, 1), Dv), 5.0, device=dev) if pool else None
@@ -378,3 +378,75 @@ def test_large_batches_take_the_grouped_expert_gemms():
         ya, yb = m._feed_forward(m.layers[0], h.cuda(), small)
         got = sum(t.double().cpu() for t in (ya, yb) if t is not None)
         torch.testing.assert_close(got, want, rtol=3e-2, atol=3e-2)
+
+
+@pytest.mark.parametrize("H,G,D,Dv,rot,window,pool,BS", [
+    (6, 3, 64, 64, 32, 44, 12, 32), (4, 2, 32, 32, 16, 24, 8, 32), (8, 2, 128, 128, 64, 100, 48, 32),
+    (2, 1, 16, 256, 0, 0, 0, 16), (4, 4, 80, 64, 16, 33, 0, 8), (3, 1, 48, 32, 48, 7, 5, 16),
+    (4, 1, 128, 128, 128, 200, 4, 32)])
+def test_attention_matrix_core_kernel(H, G, D, Dv, rot, window, pool, BS):
+    """Prompt chunks on the matrix cores against the row ops on the CPU: chunks that start in
+    the middle of a sequence, tiles cut by a chunk's end, more than one tile per chunk, leading
+    single rows of a mixed step, windows and pooled blocks that start inside a 32-key step."""
+    g = gen(H * D + window)
+    dt = torch.bfloat16
+    lens = [(400, 1), (77, 1), (300, 300), (391, 150), (33, 33), (260, 129)]   # (cached, rows)
+    nd = 2
+    NB = sum(-(-n // BS) for n, _ in lens) + 1
+    perm = torch.randperm(NB, generator=g).int()
+    mb = max(-(-n // BS) for n, _ in lens)
+    bt = torch.zeros(len(lens), mb, dtype=torch.int32)
+    kc = torch.zeros(NB, G, BS, D, dtype=dt)
+    vc = torch.zeros(NB, G, BS // 8, Dv, 8, dtype=dt)
+    PS = sops.pool_slots(BS, pool)
+    kp = torch.zeros(NB, G, max(PS, 1), D) if pool else None
+    vp = torch.zeros(NB, G, max(PS, 1), Dv) if pool else None
+    cs = sops.rotary_table_yarn(512, rot, 1000.0, None) if rot else None
+    N = H * D + G * (D + Dv)
+    o = 0
+    for b, (n, _) in enumerate(lens):       # fill the cache of every sequence from position 0
+        nbk = -(-n // BS)
+        bt[b, :nbk] = perm[o:o + nbk]
+        o += nbk
+        pos = torch.arange(n)
+        slots = bt[b][pos // BS].long() * BS + pos % BS
+        proj = torch.randn(n, N, generator=g).to(dt)
+        sops.bias_rope_cache(proj, torch.zeros(n, H, D, dtype=dt), kc, vc, pos, slots, cs, None,
+                             H, G, D, Dv, 0, H * D, H * D + G * D)
+        if pool:
+            sops.pool_cache_blocks(kc, vc, kp, vp, pos, slots, bt[b:b + 1],
+                                   torch.tensor([0, n], dtype=torch.int32), pool)
+    rows = [r for _, r in lens]
+    T = sum(rows)
+    q = torch.randn(T, H, D, generator=g).to(dt)
+    qs = torch.tensor([0] + rows).cumsum(0).int()
+    pos = torch.cat([torch.arange(n - r, n) for n, r in lens])
+    slots = torch.cat([bt[b][torch.arange(n - r, n) // BS].long() * BS + torch.arange(n - r, n) % BS
+                       for b, (n, r) in enumerate(lens)])
+    tiles = sorted((min(r - r0, 128) + n - r + r0, b, r0) for b, (n, r) in enumerate(lens)
+                   if b >= nd for r0 in range(0, r, 128))
+    tile_seq = torch.tensor([t[1] for t in tiles], dtype=torch.int32)
+    tile_row = torch.tensor([t[2] for t in tiles], dtype=torch.int32)
+    want = torch.zeros(T, H * Dv, dtype=dt)
+    sops.pooled_window_attention(want, q, kc, vc, kp, vp, bt, qs, pos, slots, 0.2, window, pool, True)
+    mv = lambda t: None if t is None else t.cuda()  # noqa: E731
+    got = torch.zeros(T, H * Dv, dtype=dt, device="cuda")
+    assert sops.pooled_mfma_ok(q.cuda(), kc.cuda(), vc.cuda())
+    sops.pooled_window_attention_prefill(got, q.cuda(), kc.cuda(), vc.cuda(), mv(kp), mv(vp),
+                                         bt.cuda(), qs.cuda(), pos.cuda(), slots.cuda(),
+                                         tile_seq.cuda(), tile_row.cuda(), 128, 0.2, window, pool,
+                                         True, first_seq=nd)
+    close(got, want, "bfloat16", scale=2.0)
+    # one query per sequence (the last position of each) plus a padding row, heads as columns
+    last = torch.tensor([r - 1 for r in torch.tensor(rows).cumsum(0).tolist()])
+    B = len(lens)
+    qd = torch.cat([q[last], torch.zeros(1, H, D, dtype=dt)])
+    posd = torch.cat([pos[last], torch.zeros(1, dtype=torch.long)])
+    slotd = torch.cat([slots[last], torch.tensor([-1])])
+    btd = torch.cat([bt, bt[:1]])
+    got = torch.full((B + 1, H * Dv), 3.0, dtype=dt, device="cuda")
+    sops.pooled_window_attention_decode(got, qd.cuda(), kc.cuda(), vc.cuda(), mv(kp), mv(vp),
+                                        btd.cuda(), posd.cuda(), slotd.cuda(), 0.2, window, pool,
+                                        True)
+    close(got[:B], want[last], "bfloat16", scale=2.0)
+    assert (got[B] == 3.0).all()                     # the padding row is left unwritten
