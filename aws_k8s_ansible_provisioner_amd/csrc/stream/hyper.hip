@@ -230,9 +230,9 @@ __global__ __launch_bounds__(256) void route_sigmoid_kernel(int32_t* __restrict_
                                                             const float* __restrict__ router, int d,
                                                             int E, int top, int groups, int keep,
                                                             int group_top) {
-  extern __shared__ float lds[];   // [d] row, [E] scores, [E] choice values, [groups] group scores
-  float* hs = lds;
-  float* sc = lds + d;
+  extern __shared__ __align__(16) float lds[];   // [d] row (padded to 4), [E] scores, [E] choice
+  float* hs = lds;                               // values, [groups] group scores
+  float* sc = lds + ((d + 3) & ~3);
   float* ch = sc + E;
   float* gs = ch + E;
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -242,7 +242,17 @@ __global__ __launch_bounds__(256) void route_sigmoid_kernel(int32_t* __restrict_
   for (int e = wave; e < E; e += 4) {
     const float* r = router + (size_t)e * d;
     float acc = 0.f;
-    for (int c = lane; c < d; c += 64) acc += hs[c] * r[c];
+    if ((d & 3) == 0 && ((uintptr_t)router & 15) == 0) {
+      float a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll 4
+      for (int c = lane * 4; c < d; c += 256) {
+        const float4 w4 = *(const float4*)(r + c), h4 = *(const float4*)(hs + c);
+        acc += h4.x * w4.x; a1 += h4.y * w4.y; a2 += h4.z * w4.z; a3 += h4.w * w4.w;
+      }
+      acc = (acc + a1) + (a2 + a3);
+    } else {
+      for (int c = lane; c < d; c += 64) acc += hs[c] * r[c];
+    }
     acc = wave_sum(acc);
     if (lane == 0) {
       const float s = 1.0f / (1.0f + expf(-acc));
@@ -339,6 +349,97 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(const ConvArgs a) {
   a.out[(size_t)t * a.C + c] = siluf(acc);
 }
 
+// four channels per thread over a tile of RB rows (kConvRows for prompt chunks, 1 for steps of
+// single rows, where every row starts from its slot anyway; C % 4 == 0, rows and pointers aligned
+// for 8- / 16-byte accesses): the weights are read once, the last taps - 1 inputs slide through
+// registers, a row costs one load and one store; at a sequence's first row of the step the
+// history comes from its slot
+constexpr int kConvRows = 16;
+
+template <typename TY>
+__global__ __launch_bounds__(256) void conv_silu_vec_kernel(const ConvArgs a, const int RB) {
+  const int c = (blockIdx.y * 256 + threadIdx.x) * 4;
+  if (c >= a.C) return;
+  const int tb = blockIdx.x * RB, te = min(a.T, tb + RB);
+  constexpr bool F32 = sizeof(TY) == 4;
+  const TY* proj = (const TY*)a.proj;
+  float bias[4], w[4][kMaxTaps], hist[kMaxTaps][4];   // hist[j]: the input taps - 1 - j rows back
+  ld4v(a.b, true, c, bias);
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+#pragma unroll
+    for (int j = 0; j < kMaxTaps; ++j) w[k][j] = j < a.taps ? a.w[(size_t)(c + k) * a.taps + j] : 0.f;
+  int b = a.q_start ? seq_of_row(a.q_start, a.B, tb) : tb;
+  int r1 = tb;                                        // forces the first row to load its history
+  int slot = -1;
+  for (int t = tb; t < te; ++t) {
+    if (t >= r1) {                                    // a new sequence (or the tile's first row)
+      int r0;
+      if (a.q_start) {
+        if (t > tb) ++b;
+        while (a.q_start[b + 1] <= t) ++b;            // empty sequences
+        r0 = a.q_start[b];
+        r1 = a.q_start[b + 1];
+      } else {
+        r0 = t;
+        r1 = t + 1;
+      }
+      slot = a.seq_slot[r0];
+      const int pos0 = (int)a.positions[r0];
+      const TY* st = (const TY*)a.state + (size_t)(slot < 0 ? 0 : slot) * (a.taps - 1) * a.C;
+#pragma unroll
+      for (int j = 0; j < kMaxTaps - 1; ++j) {
+        if (j < a.taps - 1) {
+          const int src = t - (a.taps - 1 - j);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) hist[j][k] = 0.f;
+          if (slot >= 0) {
+            if (src >= r0) {
+              ld4v(proj, F32, (size_t)src * a.proj_stride + a.off + c, hist[j]);
+            } else {
+              const int kk = src - r0;                // -1: the input just before the step
+              if (pos0 + kk >= 0) ld4v(st, F32, (size_t)(a.taps - 1 + kk) * a.C + c, hist[j]);
+            }
+          }
+        }
+      }
+    }
+    float cur[4];
+    ld4v(proj, F32, (size_t)t * a.proj_stride + a.off + c, cur);
+    float acc[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) acc[k] = bias[k];
+#pragma unroll
+    for (int j = 0; j < kMaxTaps - 1; ++j)
+      if (j < a.taps - 1) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc[k] += w[k][j] * hist[j][k];
+      }
+    float o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float wl = 0.f;
+#pragma unroll
+      for (int j = 0; j < kMaxTaps; ++j)
+        if (j == a.taps - 1) wl = w[k][j];
+      o[k] = siluf(acc[k] + wl * cur[k]);
+    }
+    if (slot >= 0) st4(a.out + (size_t)t * a.C + c, o);
+#pragma unroll
+    for (int j = 0; j < kMaxTaps - 2; ++j)
+      if (j < a.taps - 2) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) hist[j][k] = hist[j + 1][k];
+      }
+#pragma unroll
+    for (int j = 0; j < kMaxTaps - 1; ++j)
+      if (j == a.taps - 2) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) hist[j][k] = cur[k];
+      }
+  }
+}
+
 // a thread per (sequence, channel): the last taps - 1 inputs of the sequence go to its slot
 template <typename TY>
 __global__ __launch_bounds__(256) void conv_state_kernel(const ConvArgs a) {
@@ -382,54 +483,103 @@ struct ScanArgs {
   const int64_t* positions;
   const int32_t* q_start;  // [B + 1] or null
   int proj_stride, dt_off, H, V, N, G, T, B;
+  int VL;                  // state columns of a workgroup (V / VL workgroups per head)
 };
 
 constexpr int kScanTokens = 16;
 
 __host__ __device__ __forceinline__ int up4(int n) { return (n + 3) & ~3; }
 
-// One workgroup per (sequence, head).  Thread (v, part) owns column v of the R consecutive
-// state rows part R .. part R + R - 1 (NP = 256 / V parts), in registers over all rows of the
-// step.  Tokens are staged TK at a time (x, B, C, step size and decay; TK = 16 for prompt
-// chunks, 1 for steps of single rows); per token a thread updates its rows and adds its share
-// of S^T C, reading B and C from LDS four rows at a time (all lanes of a wave read the same
-// addresses); the parts' shares meet in LDS after the staged tokens.
+// One workgroup per (sequence, head, VL state columns) -- the columns of a state are independent;
+// the launcher gives a workgroup the whole head.  Thread (v, part) owns column v of the R
+// consecutive state rows part R .. part R + R - 1 (NP = 256 / VL parts), in registers over all
+// rows of the step.  Tokens are staged TK at a time (x, B, C, step size and decay; TK = 16 for
+// prompt chunks, fetched into registers one stage ahead; 1 for steps of single rows); per token
+// a thread updates its rows and adds its share of S^T C, reading B and C from LDS four rows at a
+// time (all lanes of a wave read the same addresses); the parts' shares meet in LDS after the
+// staged tokens.
 template <typename TY, int R>
 __global__ __launch_bounds__(256) void selective_scan_kernel(const ScanArgs a, const int TK) {
   extern __shared__ __align__(16) float lds[];
-  const int V = a.V, N = a.N, NP = 256 / V;
+  const int V = a.VL, N = a.N, NP = 256 / V;    // V: the columns of this workgroup
   float* xs = lds;                              // [TK][V]
   float* bs = xs + up4(TK * V);                 // [TK][N]
   float* cs = bs + up4(TK * N);                 // [TK][N]
   float* dts = cs + up4(TK * N);                // [TK] step, [TK] decay
   float* ys = dts + up4(2 * TK);                // [TK][NP][V]
-  const int b = blockIdx.x, h = blockIdx.y;
+  const int nsplit = a.V / V;
+  const int b = blockIdx.x, h = blockIdx.y / nsplit, v0 = (blockIdx.y - h * nsplit) * V;
   const int r0 = a.q_start ? a.q_start[b] : b;
   const int r1 = a.q_start ? a.q_start[b + 1] : b + 1;
   if (r1 <= r0) return;
   const int slot = a.seq_slot[r0];
   if (slot < 0) return;
   const int g = h / (a.H / a.G);
-  const int inner = a.H * V, C = inner + 2 * a.G * N;
+  const int inner = a.H * a.V, C = inner + 2 * a.G * N;
   const int tid = threadIdx.x;
   const int v = tid % V, part = tid / V;
   const int n0 = part * R;
   const bool active = part < NP && n0 < N;
   const bool vec = (N & 3) == 0 && (R & 3) == 0;
-  float* sp = a.state + ((size_t)slot * a.H + h) * N * V;
+  float* sp = a.state + ((size_t)slot * a.H + h) * N * a.V + v0;
   float S[R];
   const bool carry = a.positions[r0] > 0;
 #pragma unroll
   for (int r = 0; r < R; ++r)
-    S[r] = (carry && active && n0 + r < N) ? sp[(size_t)(n0 + r) * V + v] : 0.f;
+    S[r] = (carry && active && n0 + r < N) ? sp[(size_t)(n0 + r) * a.V + v] : 0.f;
   const float ea = expf(a.a_log[h]), dsk = a.d_skip[h], dtb = a.dt_bias[h];
   const TY* proj = (const TY*)a.proj;
+  // prompt chunks with sizes in fours: the next 16 tokens are fetched into registers (16-byte
+  // loads, all issued together) while the current 16 are computed
+  const bool vstage = TK == kScanTokens && (V & 3) == 0 && (N & 3) == 0 && (a.V & 3) == 0 &&
+                      V <= 256 && N <= 256;
+  const int V4 = V >> 2, N4 = N >> 2;
+  float4 px[4], pb[4], pc[4];
+  float pdt = 0.f;
+  auto prefetch = [&](int c0) {
+    const int nt = min(TK, r1 - c0);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = tid + 256 * u;
+      if (i < nt * V4) {
+        const int tk = i / V4, e = i - tk * V4;
+        px[u] = *(const float4*)(a.xbc + (size_t)(c0 + tk) * C + h * a.V + v0 + 4 * e);
+      }
+      if (i < nt * N4) {
+        const int tk = i / N4, e = i - tk * N4;
+        const float* row = a.xbc + (size_t)(c0 + tk) * C + inner + g * N + 4 * e;
+        pb[u] = *(const float4*)row;
+        pc[u] = *(const float4*)(row + a.G * N);
+      }
+    }
+    if (tid < nt) pdt = ldf(proj + (size_t)(c0 + tid) * a.proj_stride + a.dt_off + h);
+  };
+  if (vstage) prefetch(r0);
   for (int c0 = r0; c0 < r1; c0 += TK) {
     const int nt = min(TK, r1 - c0);
     __syncthreads();
+    if (vstage) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = tid + 256 * u;
+        if (i < nt * V4) *(float4*)(xs + 4 * i) = px[u];
+        if (i < nt * N4) {
+          *(float4*)(bs + 4 * i) = pb[u];
+          *(float4*)(cs + 4 * i) = pc[u];
+        }
+      }
+      if (tid < nt) {
+        const float z = pdt + dtb;
+        const float dt = z > 20.f ? z : log1pf(expf(z));
+        dts[tid] = dt;
+        dts[TK + tid] = expf(-ea * dt);
+      }
+      __syncthreads();
+      if (c0 + TK < r1) prefetch(c0 + TK);
+    } else {
     for (int i = tid; i < nt * V; i += 256) {
       const int tk = i / V, e = i - tk * V;
-      xs[tk * V + e] = a.xbc[(size_t)(c0 + tk) * C + h * V + e];
+      xs[tk * V + e] = a.xbc[(size_t)(c0 + tk) * C + h * a.V + v0 + e];
     }
     for (int i = tid; i < nt * N; i += 256) {
       const int tk = i / N, e = i - tk * N;
@@ -444,6 +594,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(const ScanArgs a, c
       dts[TK + tid] = expf(-ea * dt);
     }
     __syncthreads();
+    }
     if (active) {
       for (int tk = 0; tk < nt; ++tk) {
         const float dt = dts[tk], dec = dts[TK + tk];
@@ -452,6 +603,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(const ScanArgs a, c
         const float* ct = cs + tk * N + n0;
         float acc = 0.f;
         if (vec) {
+          float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;   // four chains instead of one
 #pragma unroll
           for (int r = 0; r < R; r += 4) {
             if (n0 + r < N) {
@@ -460,9 +612,13 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(const ScanArgs a, c
               S[r + 1] = dec * S[r + 1] + dx * b4.y;
               S[r + 2] = dec * S[r + 2] + dx * b4.z;
               S[r + 3] = dec * S[r + 3] + dx * b4.w;
-              acc += S[r] * c4.x + S[r + 1] * c4.y + S[r + 2] * c4.z + S[r + 3] * c4.w;
+              a0 += S[r] * c4.x;
+              a1 += S[r + 1] * c4.y;
+              a2 += S[r + 2] * c4.z;
+              a3 += S[r + 3] * c4.w;
             }
           }
+          acc = (a0 + a1) + (a2 + a3);
         } else {
 #pragma unroll
           for (int r = 0; r < R; ++r) {
@@ -482,13 +638,144 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(const ScanArgs a, c
       const int tk = i / V, e = i - tk * V;
       float acc = dsk * xs[tk * V + e];
       for (int p = 0; p < NP; ++p) acc += ys[(tk * NP + p) * V + e];
+      a.y[(size_t)(c0 + tk) * inner + h * a.V + v0 + e] = acc;
+    }
+  }
+  if (active) {
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (n0 + r < N) sp[(size_t)(n0 + r) * a.V + v] = S[r];
+  }
+}
+
+// The same recurrence with FOUR neighbouring state columns per thread (V a multiple of 4 with
+// V / 4 a power of two up to 64): thread (cg, part) owns columns 4 cg .. 4 cg + 3 of the R rows
+// part R .. part R + R - 1 (NP = 1024 / V parts).  A staged B or C value now serves four
+// columns, so a token costs a quarter of the LDS reads (the one-column form is bound by them),
+// and the state moves in 16-byte pieces.  The parts of a wave add their shares of S^T C by lane
+// exchange, the four waves' sums meet in LDS.  PRE: prompt chunks, the next 16 tokens are
+// fetched into registers while the current 16 are computed.
+template <typename TY, int R, bool PRE>
+__global__ __launch_bounds__(256) void selective_scan4_kernel(const ScanArgs a, const int TK) {
+  extern __shared__ __align__(16) float lds[];
+  const int V = a.V, N = a.N, V4 = V >> 2, N4 = N >> 2, NP = 256 / V4;
+  float* xs = lds;                              // [TK][V]
+  float* bs = xs + up4(TK * V);                 // [TK][N]
+  float* cs = bs + up4(TK * N);                 // [TK][N]
+  float* dts = cs + up4(TK * N);                // [TK] step, [TK] decay
+  float* ys = dts + up4(2 * TK);                // [TK][4][V]
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int r0 = a.q_start ? a.q_start[b] : b;
+  const int r1 = a.q_start ? a.q_start[b + 1] : b + 1;
+  if (r1 <= r0) return;
+  const int slot = a.seq_slot[r0];
+  if (slot < 0) return;
+  const int g = h / (a.H / a.G);
+  const int inner = a.H * V, C = inner + 2 * a.G * N;
+  const int tid = threadIdx.x, wave = tid >> 6;
+  const int cg = tid % V4, part = tid / V4;
+  const int n0 = part * R;
+  const bool active = n0 < N;
+  float* sp = a.state + ((size_t)slot * a.H + h) * N * V + 4 * cg;
+  float4 S[R];
+  const bool carry = a.positions[r0] > 0;
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+    S[r] = (carry && active && n0 + r < N) ? *(const float4*)(sp + (size_t)(n0 + r) * V)
+                                           : make_float4(0.f, 0.f, 0.f, 0.f);
+  const float ea = expf(a.a_log[h]), dsk = a.d_skip[h], dtb = a.dt_bias[h];
+  const TY* proj = (const TY*)a.proj;
+  float4 px[PRE ? 4 : 1], pb[PRE ? 4 : 1], pc[PRE ? 4 : 1];
+  float pdt = 0.f;
+  auto prefetch = [&](int c0) {
+    const int nt = min(TK, r1 - c0);
+#pragma unroll
+    for (int u = 0; u < (PRE ? 4 : 1); ++u) {
+      const int i = tid + 256 * u;
+      if (i < nt * V4) {
+        const int tk = i / V4, e = i - tk * V4;
+        px[u] = *(const float4*)(a.xbc + (size_t)(c0 + tk) * C + h * V + 4 * e);
+      }
+      if (i < nt * N4) {
+        const int tk = i / N4, e = i - tk * N4;
+        const float* row = a.xbc + (size_t)(c0 + tk) * C + inner + g * N + 4 * e;
+        pb[u] = *(const float4*)row;
+        pc[u] = *(const float4*)(row + a.G * N);
+      }
+    }
+    if (tid < nt) pdt = ldf(proj + (size_t)(c0 + tid) * a.proj_stride + a.dt_off + h);
+  };
+  prefetch(r0);
+  for (int c0 = r0; c0 < r1; c0 += TK) {
+    const int nt = min(TK, r1 - c0);
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < (PRE ? 4 : 1); ++u) {
+      const int i = tid + 256 * u;
+      if (i < nt * V4) *(float4*)(xs + 4 * i) = px[u];
+      if (i < nt * N4) {
+        *(float4*)(bs + 4 * i) = pb[u];
+        *(float4*)(cs + 4 * i) = pc[u];
+      }
+    }
+    if (tid < nt) {
+      const float z = pdt + dtb;
+      const float dt = z > 20.f ? z : log1pf(expf(z));
+      dts[tid] = dt;
+      dts[TK + tid] = expf(-ea * dt);
+    }
+    __syncthreads();
+    if (PRE && c0 + TK < r1) prefetch(c0 + TK);
+    for (int tk = 0; tk < nt; ++tk) {
+      const float dt = dts[tk], dec = dts[TK + tk];
+      const float4 x4 = *(const float4*)(xs + tk * V + 4 * cg);
+      const float4 dx = make_float4(dt * x4.x, dt * x4.y, dt * x4.z, dt * x4.w);
+      const float* bt = bs + tk * N + n0;
+      const float* ct = cs + tk * N + n0;
+      float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (active) {
+#pragma unroll
+        for (int r = 0; r < R; r += 4) {
+          if (n0 + r < N) {
+            const float4 b4 = *(const float4*)(bt + r), c4 = *(const float4*)(ct + r);
+            const float bb[4] = {b4.x, b4.y, b4.z, b4.w}, cc[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              S[r + q].x = dec * S[r + q].x + dx.x * bb[q];
+              S[r + q].y = dec * S[r + q].y + dx.y * bb[q];
+              S[r + q].z = dec * S[r + q].z + dx.z * bb[q];
+              S[r + q].w = dec * S[r + q].w + dx.w * bb[q];
+              acc.x += S[r + q].x * cc[q];
+              acc.y += S[r + q].y * cc[q];
+              acc.z += S[r + q].z * cc[q];
+              acc.w += S[r + q].w * cc[q];
+            }
+          }
+        }
+      }
+      // the parts of this wave (lanes V4 apart)
+      for (int o = V4; o < 64; o <<= 1) {
+        acc.x += __shfl_xor(acc.x, o, 64);
+        acc.y += __shfl_xor(acc.y, o, 64);
+        acc.z += __shfl_xor(acc.z, o, 64);
+        acc.w += __shfl_xor(acc.w, o, 64);
+      }
+      if ((tid & 63) < V4 || V4 >= 64) *(float4*)(ys + (tk * 4 + wave) * V + 4 * cg) = acc;
+    }
+    __syncthreads();
+    // V4 >= 64: a wave holds one part of 64 column groups, its sums cover columns of its own
+    for (int i = tid; i < nt * V; i += 256) {
+      const int tk = i / V, e = i - tk * V;
+      float acc = dsk * xs[tk * V + e];
+#pragma unroll
+      for (int w = 0; w < 4; ++w) acc += ys[(tk * 4 + w) * V + e];
       a.y[(size_t)(c0 + tk) * inner + h * V + e] = acc;
     }
   }
   if (active) {
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      if (n0 + r < N) sp[(size_t)(n0 + r) * V + v] = S[r];
+      if (n0 + r < N) *(float4*)(sp + (size_t)(n0 + r) * V) = S[r];
   }
 }
 
@@ -542,7 +829,7 @@ void launch_route_sigmoid(int32_t* ids, float* w, const void* h, int h_stride, b
                           const float* router, int rows, int d, int E, int top, int groups,
                           int keep, int group_top, hipStream_t s) {
   if (rows <= 0) return;
-  const size_t lds = (size_t)(d + 2 * E + groups) * sizeof(float);
+  const size_t lds = (size_t)(((d + 3) & ~3) + 2 * E + groups) * sizeof(float);
   if (f32)
     route_sigmoid_kernel<float><<<rows, 256, lds, s>>>(ids, w, (const float*)h, h_stride, router,
                                                        d, E, top, groups, keep, group_top);
@@ -557,8 +844,16 @@ void launch_conv_silu(float* out, const void* proj, int proj_stride, int off, bo
                       int taps, hipStream_t s) {
   if (T <= 0) return;
   ConvArgs a{out, proj, state, w, b, seq_slot, positions, q_start, proj_stride, off, C, taps, T, B};
-  const dim3 g1(T, (C + 255) / 256), g2(B, (C + 255) / 256);
-  if (f32) conv_silu_kernel<float><<<g1, 256, 0, s>>>(a);
+  const dim3 g1(T, (C + 255) / 256), g2(B, (C + 255) / 256), g4((T + (q_start ? kConvRows : 1) - 1) / (q_start ? kConvRows : 1), (C / 4 + 255) / 256);
+  const int RB = q_start ? kConvRows : 1;
+  const int es = f32 ? 4 : 2;
+  const bool vec = C % 4 == 0 && off % 4 == 0 && proj_stride % 4 == 0 &&
+                   (uintptr_t)proj % (4 * es) == 0 && (uintptr_t)state % (4 * es) == 0 &&
+                   (uintptr_t)out % 16 == 0 && (uintptr_t)b % 16 == 0;
+  if (vec) {
+    if (f32) conv_silu_vec_kernel<float><<<g4, 256, 0, s>>>(a, RB);
+    else conv_silu_vec_kernel<bf16><<<g4, 256, 0, s>>>(a, RB);
+  } else if (f32) conv_silu_kernel<float><<<g1, 256, 0, s>>>(a);
   else conv_silu_kernel<bf16><<<g1, 256, 0, s>>>(a);
   if (taps > 1) {
     if (f32) conv_state_kernel<float><<<g2, 256, 0, s>>>(a);
@@ -578,12 +873,42 @@ void launch_selective_scan(float* y, const float* xbc, const void* proj, int pro
                            int V, int N, int G, hipStream_t s) {
   if (T <= 0) return;
   ScanArgs a{y, xbc, proj, dt_bias, a_log, d_skip, state, seq_slot, positions, q_start,
-             proj_stride, dt_off, H, V, N, G, T, B};
-  const int NP = 256 / V, R = selective_scan_rows(V, N);
+             proj_stride, dt_off, H, V, N, G, T, B, V};
   const int TK = q_start ? kScanTokens : 1;
+  const dim3 grid(B, H);
+  // four columns per thread: V / 4 a power of two up to 64 (a wave holds whole parts), at most
+  // 64 columns per part-row of a wave, N in fours, rows of a thread in fours
+  const int V4 = V / 4;
+  const bool four = V % 4 == 0 && V4 >= 1 && V4 <= 32 && (V4 & (V4 - 1)) == 0 && N % 4 == 0 &&
+                    N <= 256;
+  if (four) {
+    const int NP = 256 / V4;
+    int R = (N + NP - 1) / NP;
+    R = (R + 3) & ~3;
+    const size_t lds = (size_t)(up4(TK * V) + 2 * up4(TK * N) + up4(2 * TK) + TK * 4 * V) *
+                       sizeof(float);
+#define AKAP_SCAN4(TY, RR)                                                          \
+  do {                                                                              \
+    if (q_start) selective_scan4_kernel<TY, RR, true><<<grid, 256, lds, s>>>(a, TK); \
+    else selective_scan4_kernel<TY, RR, false><<<grid, 256, lds, s>>>(a, TK);       \
+  } while (0)
+#define AKAP_SCAN4_R(TY)                \
+  do {                                  \
+    if (R <= 4) AKAP_SCAN4(TY, 4);      \
+    else if (R <= 8) AKAP_SCAN4(TY, 8); \
+    else AKAP_SCAN4(TY, 16);            \
+  } while (0)
+    if (R <= 16) {
+      if (f32) AKAP_SCAN4_R(float);
+      else AKAP_SCAN4_R(bf16);
+      return;
+    }
+#undef AKAP_SCAN4_R
+#undef AKAP_SCAN4
+  }
+  const int NP = 256 / V, R = selective_scan_rows(V, N);
   const size_t lds = (size_t)(up4(TK * V) + 2 * up4(TK * N) + up4(2 * TK) + TK * NP * V) *
                      sizeof(float);
-  const dim3 grid(B, H);
 #define AKAP_SCAN(TY, RR) selective_scan_kernel<TY, RR><<<grid, 256, lds, s>>>(a, TK)
 #define AKAP_SCAN_R(TY)                  \
   do {                                   \

@@ -111,12 +111,17 @@ __global__ __launch_bounds__(256) void bias_rope_cache_kernel(const RopeCachePar
 }
 
 // ------------------------------------------------------------------ pooled entries
-// one workgroup per (row, key/value head); rows that do not end a block leave at once
+// one workgroup per (RB rows, key/value head): 32 rows for large steps (few rows end a block,
+// a workgroup per row would mostly launch and leave), one otherwise; rows that do not end a
+// block are passed over
+constexpr int kPoolRows = 32;
+
 template <typename T>
-__global__ __launch_bounds__(128) void pool_cache_blocks_kernel(const PoolParams p) {
-  const int t = blockIdx.x, g = blockIdx.y;
+__global__ __launch_bounds__(128) void pool_cache_blocks_kernel(const PoolParams p, const int RB) {
+  const int g = blockIdx.y;
+  for (int t = blockIdx.x * RB; t < min(p.T, (int)(blockIdx.x + 1) * RB); ++t) {
   const int pos = (int)p.positions[t];
-  if (p.slots[t] < 0 || (pos + 1) % p.pool) return;
+  if (p.slots[t] < 0 || (pos + 1) % p.pool) continue;
   const int b = p.q_start ? seq_of_row(p.q_start, p.B, t) : t;
   const int32_t* bt = p.block_tables + (size_t)b * p.max_blocks;
   const int first = pos + 1 - p.pool;
@@ -147,6 +152,7 @@ __global__ __launch_bounds__(128) void pool_cache_blocks_kernel(const PoolParams
     }
     if (isk) p.k_pool[(((size_t)page0 * p.G + g) * p.PS + idx) * p.D + e] = acc * inv;
     else p.v_pool[(((size_t)page0 * p.G + g) * p.PS + idx) * p.Dv + e] = acc * inv;
+  }
   }
 }
 
@@ -245,9 +251,10 @@ void launch_bias_rope_cache(const RopeCacheParams& p, bool f32, hipStream_t s) {
 
 void launch_pool_cache_blocks(const PoolParams& p, bool f32, hipStream_t s) {
   if (p.T <= 0) return;
-  const dim3 grid(p.T, p.G);
-  if (f32) pool_cache_blocks_kernel<float><<<grid, 128, 0, s>>>(p);
-  else pool_cache_blocks_kernel<bf16><<<grid, 128, 0, s>>>(p);
+  const int RB = p.T >= 1024 ? kPoolRows : 1;
+  const dim3 grid((p.T + RB - 1) / RB, p.G);
+  if (f32) pool_cache_blocks_kernel<float><<<grid, 128, 0, s>>>(p, RB);
+  else pool_cache_blocks_kernel<bf16><<<grid, 128, 0, s>>>(p, RB);
 }
 
 void launch_pooled_window_attention(const PoolAttnParams& p, bool f32, hipStream_t s) {

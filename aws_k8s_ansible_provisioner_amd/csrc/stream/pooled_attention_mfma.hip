@@ -34,10 +34,12 @@ __device__ __forceinline__ bf16x8 zero8() {
 
 // DVT: 32-wide tiles of the value size.  DEC: one query per sequence (a decode step, or the
 // single rows of a mixed step): the columns of the tile are the query heads of one key/value
-// head, the four waves of the workgroup split the steps of the key range among themselves and
+// head, the eight waves of the workgroup split the steps of the key range among themselves and
 // add their shares in LDS.
+constexpr int kDecWaves = 8;
+
 template <int DVT, bool DEC>
-__global__ __launch_bounds__(256) void pooled_window_mfma_kernel(
+__global__ __launch_bounds__(DEC ? 64 * kDecWaves : 256) void pooled_window_mfma_kernel(
     const PoolAttnParams p, const int32_t* __restrict__ tile_seq,
     const int32_t* __restrict__ tile_row) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -55,7 +57,7 @@ __global__ __launch_bounds__(256) void pooled_window_mfma_kernel(
     b = t0;
     nrows = rep;                                   // columns in use: the heads of the group
     if (p.slots[t0] < 0) return;                   // a padding row (the whole workgroup)
-    for (int e = tid; e < KS * 64; e += 256) {
+    for (int e = tid; e < KS * 64; e += 64 * kDecWaves) {
       const int c = e >> 6, ln = e & 63;
       bf16x8 v = zero8();
       if ((ln & 31) < rep)
@@ -141,7 +143,7 @@ __global__ __launch_bounds__(256) void pooled_window_mfma_kernel(
   const int nbt = (P > 0 && W > 0 && plast - W + 1 > 0) ? (plast - W + 1) / P : 0;
   const int pool_steps = (nbt + 31) >> 5;
   for (int cb = 0; cb < nbt; cb += 32) {
-    if (DEC && (((cb >> 5) & 3) != wave)) continue;
+    if (DEC && ((cb >> 5) % kDecWaves != wave)) continue;
     f32x16 s;
 #pragma unroll
     for (int i = 0; i < 16; ++i) s[i] = 0.f;
@@ -188,7 +190,7 @@ __global__ __launch_bounds__(256) void pooled_window_mfma_kernel(
   // ---- window tokens, in steps aligned to 32 positions
   const int lo = W > 0 ? max(0, pos0 - W + 1) : 0;
   for (int kb = lo & ~31; kb <= plast; kb += 32) {
-    if (DEC && (((pool_steps + ((kb - (lo & ~31)) >> 5)) & 3) != wave)) continue;
+    if (DEC && ((pool_steps + ((kb - (lo & ~31)) >> 5)) % kDecWaves != wave)) continue;
     f32x16 s;
 #pragma unroll
     for (int i = 0; i < 16; ++i) s[i] = 0.f;
@@ -243,10 +245,11 @@ __global__ __launch_bounds__(256) void pooled_window_mfma_kernel(
   if (DEC) {
     // the waves' shares: maxima and sums through LDS, outputs added with LDS atomics
     __syncthreads();                               // every wave is done with the Q operands
-    float* m_s = (float*)smem;                     // [4][32]
-    float* l_s = m_s + 4 * 32;                     // [4][32]
-    float* ob = l_s + 4 * 32;                      // [Dv][32]
-    for (int e = tid; e < Dv * 32; e += 256) ob[e] = 0.f;
+    constexpr int NW = kDecWaves, NTH = 64 * kDecWaves;
+    float* m_s = (float*)smem;                     // [NW][32]
+    float* l_s = m_s + NW * 32;                    // [NW][32]
+    float* ob = l_s + NW * 32;                     // [Dv][32]
+    for (int e = tid; e < Dv * 32; e += NTH) ob[e] = 0.f;
     if (hf == 0) {
       m_s[wave * 32 + col] = m_run;
       l_s[wave * 32 + col] = l;
@@ -254,7 +257,7 @@ __global__ __launch_bounds__(256) void pooled_window_mfma_kernel(
     __syncthreads();
     float mg = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) mg = fmaxf(mg, m_s[w * 32 + col]);
+    for (int w = 0; w < NW; ++w) mg = fmaxf(mg, m_s[w * 32 + col]);
     const float f = (m_run == -INFINITY || mg == -INFINITY) ? 0.f : exp2f(m_run - mg);
     if (col < nrows && f > 0.f) {
 #pragma unroll
@@ -265,13 +268,13 @@ __global__ __launch_bounds__(256) void pooled_window_mfma_kernel(
     }
     __syncthreads();
     bf16* o = (bf16*)p.out + (size_t)t0 * p.out_stride + (size_t)g * rep * Dv;
-    for (int e = tid; e < rep * Dv; e += 256) {
+    for (int e = tid; e < rep * Dv; e += NTH) {
       const int c = e / Dv, dv = e - c * Dv;
       float mg2 = -INFINITY, lg = 0.f;
 #pragma unroll
-      for (int w = 0; w < 4; ++w) mg2 = fmaxf(mg2, m_s[w * 32 + c]);
+      for (int w = 0; w < NW; ++w) mg2 = fmaxf(mg2, m_s[w * 32 + c]);
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
+      for (int w = 0; w < NW; ++w) {
         const float mw = m_s[w * 32 + c];
         if (mw != -INFINITY) lg += l_s[w * 32 + c] * exp2f(mw - mg2);
       }
@@ -323,9 +326,10 @@ void launch_pooled_window_decode_mfma(const PoolAttnParams& p, int rows, hipStre
   if (rows <= 0) return;
   const dim3 grid(rows, p.G);
   const size_t q_bytes = (size_t)(p.D >> 4) * 64 * sizeof(bf16x8);
-  const size_t m_bytes = (size_t)(8 * 32 + p.Dv * 32) * sizeof(float);
+  const size_t m_bytes = (size_t)(2 * kDecWaves * 32 + p.Dv * 32) * sizeof(float);
   const size_t lds = q_bytes > m_bytes ? q_bytes : m_bytes;
-#define AKAP_PWD(N) pooled_window_mfma_kernel<N, true><<<grid, 256, lds, s>>>(p, nullptr, nullptr)
+#define AKAP_PWD(N) \
+  pooled_window_mfma_kernel<N, true><<<grid, 64 * kDecWaves, lds, s>>>(p, nullptr, nullptr)
   switch (p.Dv >> 5) {
     case 1: AKAP_PWD(1); break;
     case 2: AKAP_PWD(2); break;
