@@ -297,3 +297,40 @@ def test_sazepel_served_with_sampling_and_no_prefix_cache():
     hits = sum(float(ln.rsplit(" ", 1)[1]) for ln in text.splitlines()
                if ln.startswith("vllm:prefix_cache_hits_total"))
     assert hits == 0
+
+
+def test_mudepel_served_with_sampling_and_no_prefix_cache():
+    """The multi-stream design behind the same OpenAI endpoints: convolution inputs and
+    state-space states live in the scheduler's sequence slots, so a repeated prompt must give
+    the same greedy completion WITHOUT reusing cached pages, more prompts than slots are served
+    by handing slots on (each new owner starts from zeros), and sampled requests run."""
+    from aws_k8s_ansible_provisioner_amd.engine.config import EngineConfig
+    from aws_k8s_ansible_provisioner_amd.server.api_server import build_app
+
+    app, ae = build_app(EngineConfig(model="tiny-mudepel", served_model_name="m", device="cpu",
+                                     dtype="float32", max_model_len=256, max_num_seqs=2,
+                                     max_num_batched_tokens=48, block_size=32,
+                                     num_gpu_blocks=64, enable_prefix_caching=True))
+    prompt = list(range(10, 110))
+    with TestClient(app) as c:
+        outs = []
+        for _ in range(2):
+            r = c.post("/v1/completions", json={"prompt": prompt, "max_tokens": 6,
+                                                "temperature": 0.0})
+            assert r.status_code == 200, r.text
+            outs.append(r.json()["choices"][0]["text"])
+        assert outs[0] == outs[1]
+        r = c.post("/v1/completions", json={"prompt": [prompt[:20], prompt[:33], prompt[:7]],
+                                            "max_tokens": 4, "temperature": 0.0})
+        assert r.status_code == 200 and len(r.json()["choices"]) == 3
+        alone = [c.post("/v1/completions", json={"prompt": p, "max_tokens": 4,
+                                                 "temperature": 0.0}).json()["choices"][0]["text"]
+                 for p in (prompt[:20], prompt[:33], prompt[:7])]
+        assert [ch["text"] for ch in sorted(r.json()["choices"], key=lambda ch: ch["index"])] == alone
+        r = c.post("/v1/completions", json={"prompt": prompt[:50], "max_tokens": 5,
+                                            "temperature": 0.8, "top_p": 0.9, "seed": 3})
+        assert r.status_code == 200 and r.json()["usage"]["completion_tokens"] == 5
+        text = c.get("/metrics").text
+    hits = sum(float(ln.rsplit(" ", 1)[1]) for ln in text.splitlines()
+               if ln.startswith("vllm:prefix_cache_hits_total"))
+    assert hits == 0
