@@ -866,6 +866,22 @@ int selective_scan_rows(int V, int N) {
   return (N + NP - 1) / NP;
 }
 
+// four columns per thread: V / 4 a power of two up to 32 (a wave holds whole parts), N in fours
+// and at most 256, at most 32 rows per thread
+static bool scan_four(int V, int N, int* rows) {
+  const int V4 = V / 4;
+  if (!(V % 4 == 0 && V4 >= 1 && V4 <= 32 && (V4 & (V4 - 1)) == 0 && N % 4 == 0 && N <= 256))
+    return false;
+  const int NP = 256 / V4;
+  const int R = ((N + NP - 1) / NP + 3) & ~3;
+  if (rows) *rows = R;
+  return R <= 32;
+}
+
+bool selective_scan_supported(int V, int N) {
+  return V >= 1 && V <= 256 && N >= 1 && (scan_four(V, N, nullptr) || selective_scan_rows(V, N) <= 64);
+}
+
 void launch_selective_scan(float* y, const float* xbc, const void* proj, int proj_stride,
                            int dt_off, bool f32, const float* dt_bias, const float* a_log,
                            const float* d_skip, float* state, const int32_t* seq_slot,
@@ -874,19 +890,16 @@ void launch_selective_scan(float* y, const float* xbc, const void* proj, int pro
   if (T <= 0) return;
   ScanArgs a{y, xbc, proj, dt_bias, a_log, d_skip, state, seq_slot, positions, q_start,
              proj_stride, dt_off, H, V, N, G, T, B, V};
-  const int TK = q_start ? kScanTokens : 1;
+  int TK = q_start ? kScanTokens : 1;      // halved below until the staging fits 64 KB of LDS
   const dim3 grid(B, H);
-  // four columns per thread: V / 4 a power of two up to 64 (a wave holds whole parts), at most
-  // 64 columns per part-row of a wave, N in fours, rows of a thread in fours
-  const int V4 = V / 4;
-  const bool four = V % 4 == 0 && V4 >= 1 && V4 <= 32 && (V4 & (V4 - 1)) == 0 && N % 4 == 0 &&
-                    N <= 256;
-  if (four) {
-    const int NP = 256 / V4;
-    int R = (N + NP - 1) / NP;
-    R = (R + 3) & ~3;
-    const size_t lds = (size_t)(up4(TK * V) + 2 * up4(TK * N) + up4(2 * TK) + TK * 4 * V) *
-                       sizeof(float);
+  int R4 = 0;
+  if (scan_four(V, N, &R4)) {
+    const int R = R4;
+    auto need = [&](int tk) {
+      return (size_t)(up4(tk * V) + 2 * up4(tk * N) + up4(2 * tk) + tk * 4 * V) * sizeof(float);
+    };
+    while (TK > 1 && need(TK) > 65536) TK >>= 1;
+    const size_t lds = need(TK);
 #define AKAP_SCAN4(TY, RR)                                                          \
   do {                                                                              \
     if (q_start) selective_scan4_kernel<TY, RR, true><<<grid, 256, lds, s>>>(a, TK); \
@@ -894,21 +907,23 @@ void launch_selective_scan(float* y, const float* xbc, const void* proj, int pro
   } while (0)
 #define AKAP_SCAN4_R(TY)                \
   do {                                  \
-    if (R <= 4) AKAP_SCAN4(TY, 4);      \
-    else if (R <= 8) AKAP_SCAN4(TY, 8); \
-    else AKAP_SCAN4(TY, 16);            \
+    if (R <= 4) AKAP_SCAN4(TY, 4);        \
+    else if (R <= 8) AKAP_SCAN4(TY, 8);   \
+    else if (R <= 16) AKAP_SCAN4(TY, 16); \
+    else AKAP_SCAN4(TY, 32);              \
   } while (0)
-    if (R <= 16) {
-      if (f32) AKAP_SCAN4_R(float);
-      else AKAP_SCAN4_R(bf16);
-      return;
-    }
+    if (f32) AKAP_SCAN4_R(float);
+    else AKAP_SCAN4_R(bf16);
+    return;
 #undef AKAP_SCAN4_R
 #undef AKAP_SCAN4
   }
   const int NP = 256 / V, R = selective_scan_rows(V, N);
-  const size_t lds = (size_t)(up4(TK * V) + 2 * up4(TK * N) + up4(2 * TK) + TK * NP * V) *
-                     sizeof(float);
+  auto need = [&](int tk) {
+    return (size_t)(up4(tk * V) + 2 * up4(tk * N) + up4(2 * tk) + tk * NP * V) * sizeof(float);
+  };
+  while (TK > 1 && need(TK) > 65536) TK >>= 1;
+  const size_t lds = need(TK);
 #define AKAP_SCAN(TY, RR) selective_scan_kernel<TY, RR><<<grid, 256, lds, s>>>(a, TK)
 #define AKAP_SCAN_R(TY)                  \
   do {                                   \

@@ -170,7 +170,7 @@ void selective_scan(Tensor y, Tensor xbc, Tensor proj, int64_t dt_off, Tensor dt
   const int64_t T = xbc.size(0);
   TORCH_CHECK(H >= 1 && G >= 1 && H % G == 0 && V >= 1 && V <= 256 && N >= 1,
               "selective_scan: heads / groups / sizes (vdim at most 256)");
-  TORCH_CHECK(akap_stream::selective_scan_rows((int)V, (int)N) <= 64,
+  TORCH_CHECK(akap_stream::selective_scan_supported((int)V, (int)N),
               "selective_scan: state x vdim too large for the register-resident state");
   TORCH_CHECK(xbc.dim() == 2 && xbc.size(1) == H * V + 2 * G * N && y.dim() == 2 &&
                   y.size(0) == T && y.size(1) == H * V && proj.dim() == 2 && proj.size(0) == T &&
@@ -298,9 +298,9 @@ akap_stream::PoolAttnParams attn_params(Tensor& out, Tensor& q, Tensor& k_cache,
   const int64_t T = q.size(0), H = q.size(1), D = q.size(2);
   const int64_t G = k_cache.size(1), Dv = v_cache.size(3);
   TORCH_CHECK(k_cache.size(2) % 8 == 0, "attention: the block size must be a multiple of 8");
-  TORCH_CHECK(k_cache.size(3) == D && H % G == 0 && H / G <= 16 && Dv <= 256 && D <= 512 &&
-                  out.size(1) >= H * Dv, "attention: head sizes (at most 16 query heads per "
-              "key/value head, values of at most 256 entries)");
+  TORCH_CHECK(k_cache.size(3) == D && H % G == 0 && Dv <= 512 && D <= 512 &&
+                  out.size(1) >= H * Dv, "attention: head sizes (heads a multiple of the "
+              "key/value heads, keys and values of at most 512 entries)");
   TORCH_CHECK(q.scalar_type() == k_cache.scalar_type() && out.scalar_type() == q.scalar_type(),
               "attention: dtypes differ");
   TORCH_CHECK(positions.numel() >= T && slots.numel() >= T, "attention: one position per row");

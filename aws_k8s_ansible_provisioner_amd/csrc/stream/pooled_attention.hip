@@ -157,19 +157,21 @@ __global__ __launch_bounds__(128) void pool_cache_blocks_kernel(const PoolParams
 }
 
 // ------------------------------------------------------------------ attention
-// One workgroup per (row, key/value head), one wave per query head of the group.  The visible
+// One workgroup per (row, key/value head, up to 16 query heads of the group), one wave per query
+// head.  The visible
 // keys are an index range: first the pooled entries 0 .. nb-1, then the window tokens lo .. i.
 // Per piece of 64 keys a lane scores one key (its row read in 16-byte pieces), the wave updates
 // the running maximum and sum, then every lane accumulates its output dimensions over the
 // piece's values.  All waves of a workgroup walk the same range, so barriers are uniform.
-constexpr int kMaxDv = 256;
+constexpr int kMaxDv = 512;
+constexpr int kRowWaves = 16;
 
 template <typename T>
-__global__ void pooled_window_attention_kernel(const PoolAttnParams p) {
+__global__ void pooled_window_attention_kernel(const PoolAttnParams p, const int nw) {
   extern __shared__ float lds[];   // per wave: [D] query, [64] weights
   const int t = blockIdx.x, g = blockIdx.y;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int rep = p.H / p.G, h = g * rep + wave;
+  const int rep = p.H / p.G, h = g * rep + blockIdx.z * nw + wave;
   if (p.slots[t] < 0) return;
   const int b = p.q_start ? seq_of_row(p.q_start, p.B, t) : t;
   const int32_t* bt = p.block_tables + (size_t)b * p.max_blocks;
@@ -259,11 +261,14 @@ void launch_pool_cache_blocks(const PoolParams& p, bool f32, hipStream_t s) {
 
 void launch_pooled_window_attention(const PoolAttnParams& p, bool f32, hipStream_t s) {
   if (p.T <= 0) return;
+  // rep = nz * nw: every workgroup has the same number of waves (heads)
   const int rep = p.H / p.G;
-  const dim3 grid(p.T, p.G);
-  const size_t lds = (size_t)rep * (p.D + 64) * sizeof(float);
-  if (f32) pooled_window_attention_kernel<float><<<grid, 64 * rep, lds, s>>>(p);
-  else pooled_window_attention_kernel<bf16><<<grid, 64 * rep, lds, s>>>(p);
+  int nw = rep < kRowWaves ? rep : kRowWaves;
+  while (rep % nw) --nw;
+  const dim3 grid(p.T, p.G, rep / nw);
+  const size_t lds = (size_t)nw * (p.D + 64) * sizeof(float);
+  if (f32) pooled_window_attention_kernel<float><<<grid, 64 * nw, lds, s>>>(p, nw);
+  else pooled_window_attention_kernel<bf16><<<grid, 64 * nw, lds, s>>>(p, nw);
 }
 
 }  // namespace akap_stream

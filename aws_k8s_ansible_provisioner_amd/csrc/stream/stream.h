@@ -278,8 +278,10 @@ void launch_conv_silu(float* out, const void* proj, int proj_stride, int off, bo
                       void* state, const float* w, const float* b, const int32_t* seq_slot,
                       const int64_t* positions, const int32_t* q_start, int T, int B, int C,
                       int taps, hipStream_t s);
-// state rows a thread of the scan keeps in registers (at most 64)
+// state rows a thread of the one-column scan keeps in registers (at most 64); can a head of V
+// channels with N-entry states run (either form)?
 int selective_scan_rows(int V, int N);
+bool selective_scan_supported(int V, int N);
 void launch_selective_scan(float* y, const float* xbc, const void* proj, int proj_stride,
                            int dt_off, bool f32, const float* dt_bias, const float* a_log,
                            const float* d_skip, float* state, const int32_t* seq_slot,

@@ -145,7 +145,8 @@ def _conv_scan_case(dtype, H, V, N, G, taps, dev, steps, g, slots=3):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("H,V,N,G,taps", [(4, 32, 16, 4, 3), (3, 16, 8, 1, 2), (2, 64, 128, 2, 4),
-                                          (6, 48, 20, 3, 3), (1, 128, 64, 1, 1), (8, 8, 16, 8, 5)])
+                                          (6, 48, 20, 3, 3), (1, 128, 64, 1, 1), (8, 8, 16, 8, 5),
+                                          (3, 5, 3, 1, 3), (2, 128, 256, 1, 4), (2, 64, 256, 2, 2)])
 def test_conv_and_scan_kernels(dtype, H, V, N, G, taps):
     # a prompt in portions (one shorter than the taps), a mixed step, single rows, a slot used
     # again from position 0 on top of stale contents, a padding row (slot -1)
@@ -205,7 +206,7 @@ def _attention_case(dtype, H, G, D, Dv, rot, window, pool, BS, dev, steps, g, si
 @pytest.mark.parametrize("H,G,D,Dv,rot,window,pool,BS", [
     (6, 3, 64, 64, 32, 44, 12, 32), (4, 2, 32, 16, 16, 24, 8, 32), (3, 1, 20, 36, 8, 10, 3, 16),
     (8, 2, 128, 128, 64, 50, 48, 32), (2, 2, 8, 8, 0, 0, 0, 32), (4, 4, 16, 24, 16, 33, 0, 32),
-    (5, 5, 12, 7, 12, 7, 20, 16)])
+    (5, 5, 12, 7, 12, 7, 20, 16), (40, 2, 16, 8, 8, 9, 4, 16), (2, 1, 24, 300, 0, 12, 6, 16)])
 def test_attention_kernels(dtype, H, G, D, Dv, rot, window, pool, BS):
     # prompts in portions across pages and pooled blocks, a mixed step, single rows, a padding row
     steps = [[(0, 0, 70), (1, 0, 3)], [(1, 3, 1), (0, 70, 1)], [(0, 71, 59), (1, 4, 30)],
