@@ -451,3 +451,32 @@ def test_attention_matrix_core_kernel(H, G, D, Dv, rot, window, pool, BS):
                                         True)
     close(got[:B], want[last], "bfloat16", scale=2.0)
     assert (got[B] == 3.0).all()                     # the padding row is left unwritten
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mid_size_engine_against_the_cpu_ops(tmp_path, dtype):
+    """Sizes between the tiny oracle models and the benchmark's (matrix-core attention, the
+    four-column scan, 16-byte paths everywhere): the engine on the GPU against the same engine
+    on the CPU ops, over a mixed schedule with a looped span."""
+    yarn = {"factor": 8.0, "original": 128, "fast": 16.0, "slow": 2.0}
+    cfg = oracle.make_config(width=256, vocab=301, streams=2, loop=(1, 3, 2), layers=[
+        oracle.att_layer(8, 2, 64, 32, 0.11, window=96, pool=24, rot_dims=32, yarn=yarn,
+                         mlp=oracle.routed(8, 2, 96, count=4, keep=2, shared=64)),
+        oracle.ssm_layer(8, 32, 64, 2, conv=4, norm_groups=4, mlp=oracle.dense(320)),
+        oracle.att_layer(4, 4, 32, 64, 0.2, window=50, pool=7, base=5000.0,
+                         mlp=oracle.routed(6, 3, 40)),
+        oracle.ssm_layer(4, 64, 16, 1, conv=3, mlp=None)])
+    W = oracle.random_weights(cfg, seed=11)
+    path = write_model(tmp_path, cfg, W)
+    reqs = {"a": tokens(330, 301, 1), "b": tokens(140, 301, 2), "c": tokens(61, 301, 3)}
+    sched = [[("a", 200), ("b", 3)], [("a", 1), ("b", 100), ("c", 60)], [("a", 1), ("b", 1)],
+             [("a", 128), ("b", 36), ("c", 1)]]
+    want = replay(engine(path, dtype="float32", max_tokens=640, device="cpu"), reqs, sched)
+    got = replay(engine(path, dtype=dtype, max_tokens=640, device="cuda"), reqs, sched)
+    for n in reqs:
+        e = rel_err(got[n], want[n])
+        if dtype == "float32":
+            assert e.max().item() < 1e-4, f"{n}: position {int(e.argmax())} off by {e.max().item():.2e}"
+        else:
+            assert e.median().item() < 0.05 and e.max().item() < 0.5, (n, e.median().item(),
+                                                                       e.max().item())
